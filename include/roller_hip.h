@@ -1,0 +1,178 @@
+/* roller_hip.h -- C ABI of libroller_hip.so: JIT, load, launch and time the Roller fp32 GEMM on
+ * one MI355X (gfx950).
+ *
+ * The reference (NaOHCC/mlir-roller) reaches its GPU through CuPy from Python; this library is
+ * what a maintainer binds instead (ctypes, cgo, JNI ... -- plain pointers and sizes only).  Each
+ * entry point names the reference call it replaces as file:line under /root/reference/.
+ *
+ * Conventions
+ *   - every function returns an int status: 0 = success, > 0 = a hipError_t, < 0 = an RL_ERR_*
+ *     code below.  rl_last_error() returns the text for the last failure on the calling thread.
+ *   - handles are opaque pointers owned by the library; device memory is owned by whoever
+ *     allocated it (rl_malloc'd memory is freed by rl_free and by nothing else).
+ *   - one device per process (the reference pins one GPU through its environment, .env:5-6);
+ *     calls are synchronous with respect to the host except rl_launch / rl_gemm_* / rl_event_record,
+ *     which enqueue on the given stream (NULL = the default stream).
+ *   - the library is thread-safe for concurrent calls that use different plans/modules; error
+ *     text is thread-local.
+ */
+#ifndef ROLLER_HIP_H
+#define ROLLER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RL_OK 0
+#define RL_ERR_INVALID_ARG (-1001) /* bad pointer, shape, stride, alignment or tile parameter */
+#define RL_ERR_COMPILE (-1002)     /* hiprtc rejected the program; see the build log */
+#define RL_ERR_IO (-1003)          /* code-object cache could not be read or written */
+#define RL_ERR_NO_DEVICE (-1004)   /* no usable HIP device */
+
+typedef void* rl_module;
+typedef void* rl_function;
+typedef void* rl_stream;
+typedef void* rl_event;
+typedef struct rl_gemm_plan rl_gemm_plan;
+
+/* What the rTile policy needs to know about the device (mirrors the fields of TileDevice,
+ * src/arch.py:9-37, that can be read from the runtime). */
+typedef struct rl_device_props {
+  char name[128];
+  char arch[64];            /* e.g. "gfx950:sramecc+:xnack-" */
+  int compute_units;        /* 256 on MI355X */
+  int wavefront_size;       /* 64 */
+  int lds_bytes_per_block;  /* largest LDS allocation one workgroup may opt into */
+  int regs_per_block;
+  int l2_bytes;
+  int clock_khz;            /* peak engine clock */
+  int mem_clock_khz;
+  int mem_bus_bits;
+  size_t total_mem_bytes;
+} rl_device_props;
+
+/* Tile configuration of the fp32 GEMM kernel template; one field per template parameter.
+ * Replaces the (block_tile, thread_tile, rstep, pipeline_depth) tuple that the reference feeds
+ * to GEMMBuilder.build_transform_pipeline (src/roller.py:93-99). */
+typedef struct rl_gemm_config {
+  int bm, bn;      /* block tile            <- hint.block_tile                       */
+  int bk;          /* K step                <- hint.rstep                            */
+  int wm, wn;      /* wave tile             <- 64 lanes x hint.thread_tile           */
+  int mi;          /* 32: v_mfma_f32_32x32x2_f32, 16: v_mfma_f32_16x16x4_f32        */
+  int stages;      /* LDS buffers (1 or 2)  <- pipeline_depth                        */
+  int pad_a, pad_b;/* LDS row padding in floats (multiples of 4)                     */
+  int vec;         /* 4: 128-bit global accesses, 1: dword accesses (any K, N, ld)   */
+  int edge;        /* 1: ragged tiles predicated, 0: bm|M, bn|N, bk|K required       */
+  int swz;         /* bit0: XCD-contiguous tile order, bit1: panel walk              */
+  int group;       /* panel height in tiles (reference: panel-width=8, roller.py:338)*/
+  int accum;       /* 0: C = A*B, 1: C += A*B (linalg.matmul semantics, roller.py:62)*/
+} rl_gemm_config;
+
+/* ---- library / device ---------------------------------------------------------------------- */
+
+/* Selects `device` and creates the HIP context.  Idempotent.  Replaces CuPy's implicit context
+ * creation on first use (src/roller.py:532). */
+int rl_init(int device);
+
+/* Fills *out for the device chosen by rl_init.  Replaces the hard-coded device constants of
+ * src/arch.py:41-61 with values read from the runtime. */
+int rl_device_info(rl_device_props* out);
+
+/* Text of the last error raised on this thread ("" if none).  Replaces the Python exceptions
+ * that benchmark.py:55-58 catches per hint. */
+const char* rl_last_error(void);
+
+/* ---- JIT: hiprtc ---------------------------------------------------------------------------- */
+
+/* Compiles HIP source text for gfx950.  On success *code / *code_size receive a malloc'd code
+ * object.  *log (may be NULL) receives the malloc'd build log, also on failure.  Free both with
+ * rl_free_host.  Replaces Lower.lower_module (src/roller.py:468-496): MLIR -> PTX. */
+int rl_compile(const char* source, const char* name, const char* const* options, int n_options,
+               void** code, size_t* code_size, char** log);
+void rl_free_host(void* p);
+
+/* Replace cp.cuda.Module().load / get_function / funcSetAttribute(MAX_DYNAMIC_SHARED_SIZE_BYTES)
+ * (src/roller.py:504-510). */
+int rl_module_load(const void* code, rl_module* out);
+int rl_module_get_function(rl_module m, const char* name, rl_function* out);
+int rl_module_unload(rl_module m);
+int rl_func_set_max_dynamic_lds(rl_function f, int bytes);
+
+/* Launches f.  `args` holds n_args pointers, one per kernel parameter, each pointing at that
+ * parameter's value.  Replaces cuda_func(grid, block, args, shared_mem=) (src/roller.py:545-550). */
+int rl_launch(rl_function f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
+              unsigned bz, unsigned lds_bytes, rl_stream stream, void** args, int n_args);
+
+/* ---- device memory: replaces cp.random.rand / cp.zeros / .data.ptr (src/roller.py:532-534) -- */
+int rl_malloc(void** dptr, size_t bytes);
+int rl_free(void* dptr);
+int rl_memcpy_h2d(void* dst, const void* src, size_t bytes);
+int rl_memcpy_d2h(void* dst, const void* src, size_t bytes);
+int rl_memset(void* dptr, int byte_value, size_t bytes);
+
+/* ---- streams and events: replace cp.cuda.Event / get_elapsed_time (src/roller.py:514-522,580) */
+int rl_stream_create(rl_stream* out);
+int rl_stream_destroy(rl_stream s);
+int rl_event_create(rl_event* out);
+int rl_event_record(rl_event e, rl_stream s);
+int rl_event_sync(rl_event e);
+int rl_event_elapsed_ms(rl_event start, rl_event stop, float* ms);
+int rl_event_destroy(rl_event e);
+int rl_sync(void);
+
+/* ---- the GEMM path itself -------------------------------------------------------------------
+ * The kernel template is part of the library.  A plan is one compiled instance of it:
+ * Compiler(config, hint, pipeline_depth).compile() of src/roller.py:345-387. */
+
+/* The HIP source of the kernel template (NUL-terminated, owned by the library). */
+const char* rl_gemm_template_source(void);
+
+/* Checks cfg against the template's constraints without compiling.  *lds_bytes (may be NULL)
+ * receives the dynamic LDS size = stages * (bm*(bk+pad_a) + bk*(bn+pad_b)) * 4, the padded
+ * counterpart of hint.smem_cost * pipeline_depth (src/roller.py:385); *threads (may be NULL)
+ * receives 64 * (bm/wm) * (bn/wn). */
+int rl_gemm_config_check(const rl_gemm_config* cfg, int* lds_bytes, int* threads);
+
+/* Directory of the on-disk code-object cache (NULL or "" disables it).  Files are keyed by a hash
+ * of template source, options and hiprtc version.  The reference has no cache: it rebuilds every
+ * (shape, hint) from scratch (src/roller.py:358-387). */
+int rl_set_cache_dir(const char* path);
+
+/* Compiles cfg without touching a device and stores the code object in the cache directory
+ * (ahead-of-time warm-up; works on a machine that has no GPU).  *code_size may be NULL. */
+int rl_gemm_precompile(const rl_gemm_config* cfg, size_t* code_size);
+
+/* JIT-compiles (or fetches from the in-process / on-disk cache) and loads the kernel for cfg.
+ * Plans are shared: creating the same cfg twice returns the same plan.  *compile_ms (may be NULL)
+ * receives the time spent in hiprtc, 0 on a cache hit. */
+int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* compile_ms);
+int rl_gemm_plan_function(const rl_gemm_plan* plan, rl_function* out);
+int rl_gemm_plan_lds_bytes(const rl_gemm_plan* plan);
+int rl_gemm_plan_threads(const rl_gemm_plan* plan);
+/* Kernel resource usage read from the code object's metadata (-1 if unknown). */
+int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int* sgprs,
+                           int* spilled, int* scratch_bytes);
+/* Drops every plan and unloads its module. */
+int rl_gemm_plans_clear(void);
+
+/* Enqueues C = A*B (or C += A*B when cfg.accum) for row-major fp32 device matrices
+ * A[M,lda>=K], B[K,ldb>=N], C[M,ldc>=N].  Grid is (ceil(N/bn), ceil(M/bm)) as at
+ * src/roller.py:536 (the reference floors; ragged tiles are predicated here when cfg.edge).
+ * Rejects, with RL_ERR_INVALID_ARG and before anything is launched, shapes the plan was not built
+ * for: vec=4 with K, N or a leading dimension not a multiple of 4 or a base pointer not 16-byte
+ * aligned; edge=0 with a dimension that its tile does not divide.  M==0 or N==0 is a no-op;
+ * K==0 writes zeros (or leaves C when accumulating). */
+int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
+                        int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream);
+
+/* One call for hosts that do not keep plans: plan_create (cached) + plan_launch. */
+int rl_gemm_f32(const rl_gemm_config* cfg, const float* A, const float* B, float* C, int M,
+                int N, int K, int lda, int ldb, int ldc, rl_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ROLLER_HIP_H */

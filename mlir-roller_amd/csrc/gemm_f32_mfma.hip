@@ -1,0 +1,399 @@
+// fp32 GEMM kernel template for gfx950 (MI355X, CDNA4):  C[M,N] = A[M,K] * B[K,N]
+//
+// Row-major operands, fp32 MFMA with fp32 accumulators.  The file is a template in the
+// preprocessor sense: every rTile parameter arrives as a -D define from the JIT (hiprtc) or from
+// an ahead-of-time hipcc line, and one translation unit yields exactly one kernel, "gemm_kernel"
+// (the symbol name the reference loads, /root/reference/src/roller.py:499).
+//
+// It stands in for the kernel that the reference derives from its transform-dialect schedule
+// (/root/reference/src/roller.py:93-342): one workgroup per BM x BN tile of C, a serial K loop of
+// step BK (the policy's rstep), both operand tiles staged through workgroup memory with STAGES
+// buffers (the reference's pipeline_depth), accumulators held in registers across the K loop and
+// written once, and a workgroup-id remap for cache reuse (the reference swizzles in panels of 8,
+// roller.py:334-339).  What differs is everything below that level: the per-thread outer product
+// becomes a per-wave grid of MFMA blocks, and cp.async becomes register-staged prefetch.
+//
+// Parameters (all compile-time):
+//   BM, BN      block tile (rows, columns of C per workgroup)
+//   BK          K step per main-loop iteration; multiple of 4*(64/MI)
+//   WM, WN      wave tile; (BM/WM)*(BN/WN) waves of 64 lanes form the workgroup
+//   MI          32 -> v_mfma_f32_32x32x2_f32, 16 -> v_mfma_f32_16x16x4_f32
+//   STAGES      LDS buffers: 2 = double buffer (one barrier per K step), 1 = single buffer
+//   PAD_A,PAD_B extra floats per LDS row of the A tile ([BM][BK+PAD_A]) and B tile ([BK][BN+PAD_B])
+//   VEC         4 = 128-bit global accesses (needs K%4==0, N%4==0, lda/ldb/ldc%4==0 and 16-byte
+//               aligned base pointers), 1 = dword accesses with per-element predicates
+//   EDGE        1 = predicate ragged tiles (any M, N, K), 0 = host guarantees BM|M, BN|N, BK|K
+//   SWZ         workgroup-id remap: bit0 = give every XCD a contiguous run of tiles,
+//               bit1 = walk the tile grid in panels of GROUP tile rows
+//   GROUP, NXCD panel height in tiles; number of XCDs the dispatcher round-robins over
+//   ACCUM       1 = C += A*B (what linalg.matmul means, roller.py:62), 0 = C = A*B
+//
+// Layout trick that removes every LDS bank conflict and every register shuffle on the read side:
+// an MFMA sums over its k slots, and a GEMM does not care which MFMA block owns which column, so
+// both index sets may be permuted as long as A and B agree.
+//   * A stays K-contiguous in LDS.  A lane reads four consecutive k of its row with one
+//     ds_read_b128; the four values feed four consecutive MFMAs.  MFMA t therefore contracts over
+//     k = kk + 4*g + t for lane group g (g = lane / MI), and the B operand of that MFMA is read
+//     from row kk + 4*g + t.
+//   * B stays N-contiguous in LDS.  A lane reads VN consecutive columns with one ds_read and the
+//     VN values feed VN different column blocks, so block bj of a wave owns the columns
+//     wn0 + (bj/VN)*MI*VN + VN*(lane%MI) + bj%VN.  In the epilogue the same VN accumulators are
+//     adjacent in memory again and leave as one vector store.
+// Rows of LDS-A are padded so that (BK+PAD_A)/4 is odd: the 16-byte reads of lanes in consecutive
+// rows then fall into distinct bank groups.
+//
+// Summation order is fixed by (BK, MI) alone; there is no split-K and no atomics, so results are
+// bit-identical from run to run.
+
+#ifndef __HIPCC_RTC__  // hiprtc pre-includes the device runtime declarations
+#include <hip/hip_runtime.h>
+#endif
+
+#ifndef BM
+#define BM 128
+#endif
+#ifndef BN
+#define BN 128
+#endif
+#ifndef BK
+#define BK 16
+#endif
+#ifndef WM
+#define WM 64
+#endif
+#ifndef WN
+#define WN 64
+#endif
+#ifndef MI
+#define MI 32
+#endif
+#ifndef STAGES
+#define STAGES 2
+#endif
+#ifndef PAD_A
+#define PAD_A 4
+#endif
+#ifndef PAD_B
+#define PAD_B 0
+#endif
+#ifndef VEC
+#define VEC 4
+#endif
+#ifndef EDGE
+#define EDGE 1
+#endif
+#ifndef SWZ
+#define SWZ 3
+#endif
+#ifndef GROUP
+#define GROUP 8
+#endif
+#ifndef NXCD
+#define NXCD 8
+#endif
+#ifndef ACCUM
+#define ACCUM 0
+#endif
+
+#define NWM (BM / WM)
+#define NWN (BN / WN)
+#define NWAVES (NWM * NWN)
+#define NT (64 * NWAVES)
+#define TM (WM / MI)
+#define TN (WN / MI)
+#define KG (64 / MI)       /* lane groups along k inside one MFMA (= its k extent) */
+#define KSUPER (4 * KG)    /* k covered by the four MFMAs fed from one 128-bit A read */
+#define VN (TN >= 4 ? 4 : TN)
+#define NVB (TN / VN)
+#define LDA_S (BK + PAD_A)
+#define LDB_S (BN + PAD_B)
+#define A_STAGE (BM * LDA_S)
+#define B_STAGE (BK * LDB_S)
+#define STAGE_FLOATS (A_STAGE + B_STAGE)
+#define A_UNITS (BM * BK / 4)
+#define B_UNITS (BK * BN / 4)
+#define A_PER_T ((A_UNITS + NT - 1) / NT)
+#define B_PER_T ((B_UNITS + NT - 1) / NT)
+#define OOB_OFFSET 0x80000000u
+
+static_assert(MI == 32 || MI == 16, "MI selects v_mfma_f32_32x32x2_f32 or v_mfma_f32_16x16x4_f32");
+static_assert(BM % WM == 0 && BN % WN == 0, "wave tile must divide block tile");
+static_assert(WM % MI == 0 && WN % MI == 0, "MFMA block must divide wave tile");
+static_assert(TN == 1 || TN == 2 || TN % 4 == 0, "column blocks per wave: 1, 2 or a multiple of 4");
+static_assert(BK % KSUPER == 0, "BK must be a multiple of 4*(64/MI)");
+static_assert(PAD_A % 4 == 0 && PAD_B % 4 == 0, "LDS rows stay 16-byte aligned");
+static_assert(NT <= 1024, "at most 16 waves per workgroup");
+static_assert(STAGES == 1 || STAGES == 2, "one or two LDS buffers");
+static_assert(VEC == 4 || VEC == 1, "global access width");
+static_assert(STAGES * STAGE_FLOATS * 4 <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
+
+typedef float v2f __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+#if MI == 32
+typedef v16f acc_t;
+#define ACC_REGS 16
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x2f32((a), (b), (c), 0, 0, 0)
+// accumulator register r of lane group g holds row 8*(r/4) + 4*g + r%4 of the 32x32 block
+#define ACC_ROW(r, g) (8 * ((r) / 4) + 4 * (g) + (r) % 4)
+#else
+typedef v4f acc_t;
+#define ACC_REGS 4
+#define MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x4f32((a), (b), (c), 0, 0, 0)
+// accumulator register r of lane group g holds row 4*g + r of the 16x16 block
+#define ACC_ROW(r, g) (4 * (g) + (r))
+#endif
+
+#if VN == 4
+typedef v4f bvec_t;
+#elif VN == 2
+typedef v2f bvec_t;
+#else
+typedef float bvec_t;
+#endif
+
+#define DEV static __device__ __forceinline__
+
+// Raw buffer resource over [base, base+bytes): loads beyond it return 0, stores beyond it are
+// dropped.  Word 3 = 0x00020000 is the 32-bit raw data format on gfx9-family targets.
+DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* base, long bytes) {
+  int n = bytes <= 0 ? 0 : (bytes > 0x7fffffffL ? 0x7fffffff : (int)bytes);
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, n, 0x00020000);
+}
+
+DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool p2, bool p3) {
+#if VEC == 4
+  (void)p1; (void)p2; (void)p3;
+  return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, p0 ? off : OOB_OFFSET, 0, 0));
+#else
+  v4f v;
+  v.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p0 ? off : OOB_OFFSET, 0, 0));
+  v.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p1 ? off + 4 : OOB_OFFSET, 0, 0));
+  v.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p2 ? off + 8 : OOB_OFFSET, 0, 0));
+  v.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p3 ? off + 12 : OOB_OFFSET, 0, 0));
+  return v;
+#endif
+}
+
+// Maps the hardware workgroup id to a tile of C.
+DEV void tile_of_workgroup(int nbm, int nbn, int& tile_m, int& tile_n) {
+  int pid = blockIdx.y * gridDim.x + blockIdx.x;
+  const int npid = nbm * nbn;
+#if SWZ & 1
+  // Workgroups are dealt to the XCDs round-robin; undo that so that XCD x works on one
+  // contiguous run of the tile order and its L2 sees neighbouring tiles.
+  {
+    const int per = (npid + NXCD - 1) / NXCD;
+    int tall = npid % NXCD;
+    if (tall == 0) tall = NXCD;
+    const int xcd = pid % NXCD, loc = pid / NXCD;
+    pid = xcd < tall ? xcd * per + loc : tall * per + (xcd - tall) * (per - 1) + loc;
+  }
+#endif
+#if SWZ & 2
+  {
+    const int width = GROUP * nbn;
+    const int first_m = (pid / width) * GROUP;
+    const int rows = nbm - first_m < GROUP ? nbm - first_m : GROUP;
+    tile_m = first_m + (pid % width) % rows;
+    tile_n = (pid % width) / rows;
+  }
+#else
+  tile_m = pid / nbn;
+  tile_n = pid % nbn;
+#endif
+}
+
+extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
+    const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
+    int M, int N, int K, int lda, int ldb, int ldc) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+
+  const int tid = threadIdx.y * blockDim.x + threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / NWN) * WM;
+  const int wn0 = (wave % NWN) * WN;
+  const int lr = lane % MI;  // row of A / column slot of B inside an MFMA block
+  const int lg = lane / MI;  // k group inside an MFMA
+
+  const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
+  int tile_m, tile_n;
+  tile_of_workgroup(nbm, nbn, tile_m, tile_n);
+  if (tile_m >= nbm || tile_n >= nbn) return;  // launch wider than the tile grid
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  // ---- global -> register staging: per-thread loop-invariant offsets ----
+  unsigned a_goff[A_PER_T], b_goff[B_PER_T];
+  int a_soff[A_PER_T], b_soff[B_PER_T];
+  int a_kcol[A_PER_T], b_krow[B_PER_T];
+  bool a_ok[A_PER_T], b_ok[B_PER_T][4];
+#pragma unroll
+  for (int i = 0; i < A_PER_T; ++i) {
+    const int u = tid + i * NT;
+    const int row = u / (BK / 4), c = u % (BK / 4);
+    a_goff[i] = (unsigned)(row * lda + c * 4) * 4u;
+    a_soff[i] = row * LDA_S + c * 4;
+    a_kcol[i] = c * 4;
+    a_ok[i] = (A_UNITS % NT == 0 || u < A_UNITS) && (!EDGE || m0 + row < M);
+  }
+#pragma unroll
+  for (int i = 0; i < B_PER_T; ++i) {
+    const int u = tid + i * NT;
+    const int krow = u / (BN / 4), c = u % (BN / 4);
+    b_goff[i] = (unsigned)(krow * ldb + c * 4) * 4u;
+    b_soff[i] = krow * LDB_S + c * 4;
+    b_krow[i] = krow;
+    const bool in = (B_UNITS % NT == 0 || u < B_UNITS);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b_ok[i][e] = in && (!EDGE || n0 + c * 4 + e < N);
+  }
+
+  const float* Ag = A + (long)m0 * lda;
+  const float* Bg = B + n0;
+  long a_rem = ((long)(M - m0 - 1) * lda + K) * 4;        // valid bytes from Ag to the end of A
+  long b_rem = ((long)(K - 1) * ldb + (N - n0)) * 4;      // valid bytes from Bg to the end of B
+
+  v4f ra[A_PER_T], rb[B_PER_T];
+
+  auto fetch = [&](int kt) {
+    const int k0 = kt * BK;
+    const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, a_rem - (long)k0 * 4);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + (long)k0 * ldb, b_rem - (long)k0 * ldb * 4);
+#pragma unroll
+    for (int i = 0; i < A_PER_T; ++i) {
+      const int k = k0 + a_kcol[i];
+      ra[i] = load_unit(ar, a_goff[i],
+                        a_ok[i] && (!EDGE || k + 0 < K), a_ok[i] && (!EDGE || k + 1 < K),
+                        a_ok[i] && (!EDGE || k + 2 < K), a_ok[i] && (!EDGE || k + 3 < K));
+    }
+#pragma unroll
+    for (int i = 0; i < B_PER_T; ++i) {
+      const bool kin = !EDGE || k0 + b_krow[i] < K;
+      rb[i] = load_unit(br, b_goff[i], b_ok[i][0] && kin, b_ok[i][1] && kin, b_ok[i][2] && kin,
+                        b_ok[i][3] && kin);
+    }
+  };
+
+  auto stash = [&](int stage) {
+    float* As = lds + stage * STAGE_FLOATS;
+    float* Bs = As + A_STAGE;
+#pragma unroll
+    for (int i = 0; i < A_PER_T; ++i)
+      if (A_UNITS % NT == 0 || tid + i * NT < A_UNITS) *(v4f*)&As[a_soff[i]] = ra[i];
+#pragma unroll
+    for (int i = 0; i < B_PER_T; ++i)
+      if (B_UNITS % NT == 0 || tid + i * NT < B_UNITS) *(v4f*)&Bs[b_soff[i]] = rb[i];
+  };
+
+  acc_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < ACC_REGS; ++r) acc[i][j][r] = 0.0f;
+
+  const int a_frag = (wm0 + lr) * LDA_S + 4 * lg;   // + bi*MI*LDA_S + kk
+  const int b_frag = (4 * lg) * LDB_S + wn0 + VN * lr;  // + (kk+t)*LDB_S + v*MI*VN
+
+  auto multiply = [&](int stage) {
+    const float* As = lds + stage * STAGE_FLOATS;
+    const float* Bs = As + A_STAGE;
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += KSUPER) {
+      v4f af[TM];
+#pragma unroll
+      for (int bi = 0; bi < TM; ++bi) af[bi] = *(const v4f*)&As[a_frag + bi * MI * LDA_S + kk];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        bvec_t bf[NVB];
+#pragma unroll
+        for (int v = 0; v < NVB; ++v)
+          bf[v] = *(const bvec_t*)&Bs[b_frag + (kk + t) * LDB_S + v * MI * VN];
+#pragma unroll
+        for (int bi = 0; bi < TM; ++bi)
+#pragma unroll
+          for (int bj = 0; bj < TN; ++bj) {
+#if VN == 1
+            const float bval = bf[bj];
+#else
+            const float bval = bf[bj / VN][bj % VN];
+#endif
+            acc[bi][bj] = MFMA(af[bi][t], bval, acc[bi][bj]);
+          }
+      }
+    }
+  };
+
+  // ---- main loop ----
+  const int KT = (K + BK - 1) / BK;
+  if (KT > 0) {
+    fetch(0);
+    stash(0);
+  }
+  __syncthreads();
+  for (int kt = 0; kt < KT; ++kt) {
+    const bool more = kt + 1 < KT;
+#if STAGES == 2
+    const int cur = kt & 1;
+    if (more) fetch(kt + 1);
+    multiply(cur);
+    if (more) stash(cur ^ 1);
+    __syncthreads();
+#else
+    if (more) fetch(kt + 1);
+    multiply(0);
+    __syncthreads();
+    if (more) stash(0);
+    __syncthreads();
+#endif
+  }
+
+  // ---- epilogue: every accumulator leaves once ----
+  float* Cg = C + (long)m0 * ldc + n0;
+  const __amdgpu_buffer_rsrc_t cr = make_rsrc(Cg, ((long)(M - m0 - 1) * ldc + (N - n0)) * 4);
+#pragma unroll
+  for (int bi = 0; bi < TM; ++bi)
+#pragma unroll
+    for (int r = 0; r < ACC_REGS; ++r) {
+      const int row = wm0 + bi * MI + ACC_ROW(r, lg);
+      const bool rok = !EDGE || m0 + row < M;
+#pragma unroll
+      for (int v = 0; v < NVB; ++v) {
+        const int col = wn0 + v * MI * VN + VN * lr;
+        const unsigned off = (unsigned)(row * ldc + col) * 4u;
+        float o[VN];
+#pragma unroll
+        for (int e = 0; e < VN; ++e) o[e] = acc[bi][v * VN + e][r];
+#if VEC == 4 && VN == 4
+        const unsigned po = rok && (!EDGE || n0 + col < N) ? off : OOB_OFFSET;
+        v4f out = {o[0], o[1], o[2], o[3]};
+#if ACCUM
+        out += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(cr, po, 0, 0));
+#endif
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, out), cr, po, 0, 0);
+#elif VEC == 4 && VN == 2
+        const unsigned po = rok && (!EDGE || n0 + col < N) ? off : OOB_OFFSET;
+        v2f out = {o[0], o[1]};
+#if ACCUM
+        out += __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(cr, po, 0, 0));
+#endif
+        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, out), cr, po, 0, 0);
+#else
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+          const unsigned po = rok && (!EDGE || n0 + col + e < N) ? off + 4u * e : OOB_OFFSET;
+          float out = o[e];
+#if ACCUM
+          out += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, po, 0, 0));
+#endif
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), cr, po, 0, 0);
+        }
+#endif
+      }
+    }
+}

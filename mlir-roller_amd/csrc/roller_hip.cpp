@@ -1,0 +1,638 @@
+// libroller_hip.so -- host side of the Roller fp32 GEMM path on MI355X: hiprtc JIT of the kernel
+// template, a code-object cache (in process and on disk), module load / launch, and the small
+// set of memory, stream and event calls a benchmark needs.  Declarations and the reference
+// calls they replace: include/roller_hip.h.
+//
+// Host-only translation unit (no device code): the kernel template is pulled in as text with
+// .incbin and handed to hiprtc at run time.
+
+#include "roller_hip.h"
+
+#include <hip/hip_runtime_api.h>
+#include <hip/hiprtc.h>
+
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#ifndef RL_TEMPLATE_PATH
+#error "build with -DRL_TEMPLATE_PATH=\"<path to gemm_f32_mfma.hip>\""
+#endif
+
+// The kernel template, byte for byte, NUL-terminated.
+__asm__(
+    ".section .rodata\n"
+    ".global rl_gemm_template_begin\n"
+    "rl_gemm_template_begin:\n"
+    ".incbin \"" RL_TEMPLATE_PATH "\"\n"
+    ".byte 0\n"
+    ".previous\n");
+extern "C" const char rl_gemm_template_begin[];
+
+namespace {
+
+thread_local std::string g_error;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[2048];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_error = buf;
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail((int)e, "%s: %s (hipError %d)", what, hipGetErrorString(e), (int)e);
+}
+
+#define HIP_TRY(expr)                            \
+  do {                                           \
+    hipError_t e_ = (expr);                      \
+    if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+  } while (0)
+
+std::mutex g_mutex;  // guards everything below
+bool g_ready = false;
+int g_device = -1;
+std::string g_cache_dir;
+
+struct Plan {
+  rl_gemm_config cfg;
+  hipModule_t module = nullptr;
+  hipFunction_t func = nullptr;
+  int lds_bytes = 0;
+  int threads = 0;
+  int vgprs = -1, agprs = -1, sgprs = -1, spilled = -1, scratch = -1;
+};
+
+}  // namespace
+
+struct rl_gemm_plan : Plan {};
+
+namespace {
+
+std::map<std::string, rl_gemm_plan*> g_plans;
+
+uint64_t fnv1a(const void* data, size_t n, uint64_t h) {
+  const unsigned char* p = (const unsigned char*)data;
+  for (size_t i = 0; i < n; ++i) {
+    h ^= p[i];
+    h *= 1099511628211ull;
+  }
+  return h;
+}
+
+// Same constraints as the static_asserts of the template, reported as text instead of as a
+// compiler diagnostic.
+int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
+  if (c.mi != 32 && c.mi != 16) return fail(RL_ERR_INVALID_ARG, "mi must be 32 or 16, got %d", c.mi);
+  if (c.bm <= 0 || c.bn <= 0 || c.bk <= 0 || c.wm <= 0 || c.wn <= 0)
+    return fail(RL_ERR_INVALID_ARG, "tile sizes must be positive");
+  if (c.bm % c.wm || c.bn % c.wn)
+    return fail(RL_ERR_INVALID_ARG, "wave tile %dx%d does not divide block tile %dx%d", c.wm, c.wn, c.bm, c.bn);
+  if (c.wm % c.mi || c.wn % c.mi)
+    return fail(RL_ERR_INVALID_ARG, "MFMA block %d does not divide wave tile %dx%d", c.mi, c.wm, c.wn);
+  const int tn = c.wn / c.mi;
+  if (!(tn == 1 || tn == 2 || tn % 4 == 0))
+    return fail(RL_ERR_INVALID_ARG, "wn/mi must be 1, 2 or a multiple of 4, got %d", tn);
+  if (c.bn % 4) return fail(RL_ERR_INVALID_ARG, "bn must be a multiple of 4");
+  const int ksuper = 4 * (64 / c.mi);
+  if (c.bk % ksuper) return fail(RL_ERR_INVALID_ARG, "bk must be a multiple of %d for mi=%d, got %d", ksuper, c.mi, c.bk);
+  if (c.pad_a < 0 || c.pad_b < 0 || c.pad_a % 4 || c.pad_b % 4)
+    return fail(RL_ERR_INVALID_ARG, "pad_a/pad_b must be non-negative multiples of 4");
+  if (c.stages != 1 && c.stages != 2) return fail(RL_ERR_INVALID_ARG, "stages must be 1 or 2, got %d", c.stages);
+  if (c.vec != 4 && c.vec != 1) return fail(RL_ERR_INVALID_ARG, "vec must be 4 or 1, got %d", c.vec);
+  if ((c.edge | 1) != 1 || (c.accum | 1) != 1) return fail(RL_ERR_INVALID_ARG, "edge and accum are 0 or 1");
+  if (c.swz < 0 || c.swz > 3) return fail(RL_ERR_INVALID_ARG, "swz is a 2-bit mask");
+  if ((c.swz & 2) && c.group <= 0) return fail(RL_ERR_INVALID_ARG, "group must be positive");
+  const int nt = 64 * (c.bm / c.wm) * (c.bn / c.wn);
+  if (nt > 1024) return fail(RL_ERR_INVALID_ARG, "%d threads per workgroup exceed 1024", nt);
+  const long lds = (long)c.stages * ((long)c.bm * (c.bk + c.pad_a) + (long)c.bk * (c.bn + c.pad_b)) * 4;
+  if (lds > 160 * 1024) return fail(RL_ERR_INVALID_ARG, "%ld bytes of LDS exceed the 160 KB of a CU", lds);
+  if (lds_bytes) *lds_bytes = (int)lds;
+  if (threads) *threads = nt;
+  return RL_OK;
+}
+
+std::vector<std::string> config_options(const rl_gemm_config& c) {
+  std::vector<std::string> o;
+  auto def = [&](const char* k, int v) { o.push_back(std::string("-D") + k + "=" + std::to_string(v)); };
+  def("BM", c.bm); def("BN", c.bn); def("BK", c.bk); def("WM", c.wm); def("WN", c.wn); def("MI", c.mi);
+  def("STAGES", c.stages); def("PAD_A", c.pad_a); def("PAD_B", c.pad_b); def("VEC", c.vec);
+  def("EDGE", c.edge); def("SWZ", c.swz); def("GROUP", c.group > 0 ? c.group : 1); def("ACCUM", c.accum);
+  return o;
+}
+
+std::string config_key(const rl_gemm_config& c) {
+  std::string k;
+  for (const std::string& s : config_options(c)) k += s + " ";
+  return k;
+}
+
+int compile(const char* source, const char* name, const std::vector<std::string>& user_opts,
+            std::vector<char>* code, std::string* log) {
+  // Fixed part of the command line: the one target this library serves, and no packed-fp32
+  // instruction selection.
+  std::vector<std::string> all = {"--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature",
+                                  "-Xclang", "-packed-fp32-ops"};
+  all.insert(all.end(), user_opts.begin(), user_opts.end());
+  std::vector<const char*> argv;
+  for (const std::string& s : all) argv.push_back(s.c_str());
+
+  hiprtcProgram prog = nullptr;
+  hiprtcResult r = hiprtcCreateProgram(&prog, source, name ? name : "kernel.hip", 0, nullptr, nullptr);
+  if (r != HIPRTC_SUCCESS) return fail(RL_ERR_COMPILE, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+  r = hiprtcCompileProgram(prog, (int)argv.size(), argv.data());
+  size_t log_size = 0;
+  if (hiprtcGetProgramLogSize(prog, &log_size) == HIPRTC_SUCCESS && log_size > 1 && log) {
+    log->resize(log_size);
+    hiprtcGetProgramLog(prog, &(*log)[0]);
+    while (!log->empty() && log->back() == '\0') log->pop_back();
+  }
+  if (r != HIPRTC_SUCCESS) {
+    hiprtcDestroyProgram(&prog);
+    return fail(RL_ERR_COMPILE, "hiprtcCompileProgram: %s\n%s", hiprtcGetErrorString(r), log ? log->c_str() : "");
+  }
+  size_t n = 0;
+  r = hiprtcGetCodeSize(prog, &n);
+  if (r == HIPRTC_SUCCESS) {
+    code->resize(n);
+    r = hiprtcGetCode(prog, code->data());
+  }
+  hiprtcDestroyProgram(&prog);
+  if (r != HIPRTC_SUCCESS || code->empty())
+    return fail(RL_ERR_COMPILE, "hiprtcGetCode: %s", hiprtcGetErrorString(r));
+  return RL_OK;
+}
+
+std::string cache_path(const rl_gemm_config& c) {
+  if (g_cache_dir.empty()) return "";
+  int major = 0, minor = 0;
+  hiprtcVersion(&major, &minor);
+  const std::string key = config_key(c) + "|hiprtc " + std::to_string(major) + "." + std::to_string(minor);
+  uint64_t h1 = fnv1a(rl_gemm_template_begin, strlen(rl_gemm_template_begin), 14695981039346656037ull);
+  h1 = fnv1a(key.data(), key.size(), h1);
+  uint64_t h2 = fnv1a(key.data(), key.size(), 0x9e3779b97f4a7c15ull);
+  h2 = fnv1a(rl_gemm_template_begin, strlen(rl_gemm_template_begin), h2);
+  char name[64];
+  snprintf(name, sizeof name, "gemm_%016llx%016llx.hsaco", (unsigned long long)h1, (unsigned long long)h2);
+  return g_cache_dir + "/" + name;
+}
+
+bool read_file(const std::string& path, std::vector<char>* out) {
+  FILE* f = fopen(path.c_str(), "rb");
+  if (!f) return false;
+  fseek(f, 0, SEEK_END);
+  long n = ftell(f);
+  fseek(f, 0, SEEK_SET);
+  bool ok = n > 0;
+  if (ok) {
+    out->resize((size_t)n);
+    ok = fread(out->data(), 1, (size_t)n, f) == (size_t)n;
+  }
+  fclose(f);
+  return ok;
+}
+
+// Write-then-rename so that a concurrent reader never sees half a file.
+bool write_file(const std::string& path, const std::vector<char>& data) {
+  const std::string tmp = path + ".tmp" + std::to_string((long)getpid());
+  FILE* f = fopen(tmp.c_str(), "wb");
+  if (!f) return false;
+  bool ok = fwrite(data.data(), 1, data.size(), f) == data.size();
+  ok = (fclose(f) == 0) && ok;
+  if (ok) ok = rename(tmp.c_str(), path.c_str()) == 0;
+  if (!ok) unlink(tmp.c_str());
+  return ok;
+}
+
+// Code object for cfg: from the disk cache if present, otherwise compiled (and then cached).
+int code_for(const rl_gemm_config& c, std::vector<char>* code, float* compile_ms) {
+  if (compile_ms) *compile_ms = 0.0f;
+  const std::string path = cache_path(c);
+  if (!path.empty() && read_file(path, code)) return RL_OK;
+  std::string log;
+  const auto t0 = std::chrono::steady_clock::now();
+  int rc = compile(rl_gemm_template_begin, "gemm_f32_mfma.hip", config_options(c), code, &log);
+  if (rc != RL_OK) return rc;
+  if (compile_ms)
+    *compile_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  if (!path.empty() && !write_file(path, *code)) {
+    // A read-only cache directory is not an error for the caller: the kernel is in memory.
+    g_error = "code-object cache not writable: " + path;
+  }
+  return RL_OK;
+}
+
+// Reads an unsigned integer that follows `key` in the msgpack metadata note of a code object.
+int metadata_int(const std::vector<char>& code, const char* key) {
+  const size_t klen = strlen(key);
+  for (size_t i = 0; i + klen + 1 < code.size(); ++i) {
+    if (memcmp(&code[i], key, klen) != 0) continue;
+    const unsigned char* p = (const unsigned char*)&code[i + klen];
+    const size_t left = code.size() - (i + klen);
+    if (p[0] <= 0x7f) return p[0];
+    if (p[0] == 0xcc && left >= 2) return p[1];
+    if (p[0] == 0xcd && left >= 3) return (p[1] << 8) | p[2];
+    if (p[0] == 0xce && left >= 5) return (int)(((unsigned)p[1] << 24) | (p[2] << 16) | (p[3] << 8) | p[4]);
+  }
+  return -1;
+}
+
+// Workgroups that want more than 64 KB of dynamic LDS opt in per function.  The runtime keys this
+// attribute by host-side kernel stubs; for a function that came from hipModuleGetFunction it may
+// answer "invalid device function", which means that no opt-in exists for module functions and
+// the launch itself is the check.  Only that answer is tolerated.
+int opt_in_lds(hipFunction_t f, int bytes) {
+  hipError_t e = hipFuncSetAttribute((const void*)f, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) return RL_OK;
+  if (e == hipErrorInvalidDeviceFunction) {
+    (void)hipGetLastError();  // do not leave a sticky error for the next call
+    return RL_OK;
+  }
+  return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+}
+
+int ensure_ready() {
+  if (!g_ready) return fail(RL_ERR_NO_DEVICE, "rl_init has not been called (or failed)");
+  return RL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rl_init(int device) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (g_ready && g_device == device) return RL_OK;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0)
+    return fail(RL_ERR_NO_DEVICE, "no HIP device visible (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+  if (device < 0 || device >= count)
+    return fail(RL_ERR_INVALID_ARG, "device %d out of range (0..%d)", device, count - 1);
+  HIP_TRY(hipSetDevice(device));
+  HIP_TRY(hipFree(nullptr));  // forces context creation
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(RL_ERR_NO_DEVICE, "device %d is %s; this library is built for gfx950 (MI355X) only", device, prop.gcnArchName);
+  g_device = device;
+  g_ready = true;
+  return RL_OK;
+}
+
+int rl_device_info(rl_device_props* out) {
+  if (!out) return fail(RL_ERR_INVALID_ARG, "out is NULL");
+  int rc = ensure_ready();
+  if (rc) return rc;
+  hipDeviceProp_t p;
+  HIP_TRY(hipGetDeviceProperties(&p, g_device));
+  memset(out, 0, sizeof *out);
+  snprintf(out->name, sizeof out->name, "%s", p.name);
+  snprintf(out->arch, sizeof out->arch, "%s", p.gcnArchName);
+  out->compute_units = p.multiProcessorCount;
+  out->wavefront_size = p.warpSize;
+  out->lds_bytes_per_block = (int)p.sharedMemPerBlockOptin > 0 ? (int)p.sharedMemPerBlockOptin : (int)p.sharedMemPerBlock;
+  out->regs_per_block = p.regsPerBlock;
+  out->l2_bytes = p.l2CacheSize;
+  out->clock_khz = p.clockRate;
+  out->mem_clock_khz = p.memoryClockRate;
+  out->mem_bus_bits = p.memoryBusWidth;
+  out->total_mem_bytes = p.totalGlobalMem;
+  return RL_OK;
+}
+
+const char* rl_last_error(void) { return g_error.c_str(); }
+
+int rl_compile(const char* source, const char* name, const char* const* options, int n_options,
+               void** code, size_t* code_size, char** log) {
+  if (log) *log = nullptr;
+  if (!source || !code || !code_size || n_options < 0 || (n_options > 0 && !options))
+    return fail(RL_ERR_INVALID_ARG, "rl_compile: NULL argument");
+  *code = nullptr;
+  *code_size = 0;
+  std::vector<std::string> opts;
+  for (int i = 0; i < n_options; ++i) opts.push_back(options[i] ? options[i] : "");
+  std::vector<char> obj;
+  std::string text;
+  int rc = compile(source, name, opts, &obj, &text);
+  if (log) {
+    *log = (char*)malloc(text.size() + 1);
+    if (*log) memcpy(*log, text.c_str(), text.size() + 1);
+  }
+  if (rc != RL_OK) return rc;
+  *code = malloc(obj.size());
+  if (!*code) return fail(RL_ERR_IO, "out of host memory");
+  memcpy(*code, obj.data(), obj.size());
+  *code_size = obj.size();
+  return RL_OK;
+}
+
+void rl_free_host(void* p) { free(p); }
+
+int rl_module_load(const void* code, rl_module* out) {
+  if (!code || !out) return fail(RL_ERR_INVALID_ARG, "rl_module_load: NULL argument");
+  int rc = ensure_ready();
+  if (rc) return rc;
+  hipModule_t m = nullptr;
+  HIP_TRY(hipModuleLoadData(&m, code));
+  *out = m;
+  return RL_OK;
+}
+
+int rl_module_get_function(rl_module m, const char* name, rl_function* out) {
+  if (!m || !name || !out) return fail(RL_ERR_INVALID_ARG, "rl_module_get_function: NULL argument");
+  hipFunction_t f = nullptr;
+  HIP_TRY(hipModuleGetFunction(&f, (hipModule_t)m, name));
+  *out = f;
+  return RL_OK;
+}
+
+int rl_module_unload(rl_module m) {
+  if (!m) return RL_OK;
+  HIP_TRY(hipModuleUnload((hipModule_t)m));
+  return RL_OK;
+}
+
+int rl_func_set_max_dynamic_lds(rl_function f, int bytes) {
+  if (!f || bytes < 0) return fail(RL_ERR_INVALID_ARG, "rl_func_set_max_dynamic_lds: bad argument");
+  if (bytes > 160 * 1024) return fail(RL_ERR_INVALID_ARG, "%d bytes of LDS exceed the 160 KB of a CU", bytes);
+  return opt_in_lds((hipFunction_t)f, bytes);
+}
+
+int rl_launch(rl_function f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
+              unsigned bz, unsigned lds_bytes, rl_stream stream, void** args, int n_args) {
+  if (!f || (n_args > 0 && !args)) return fail(RL_ERR_INVALID_ARG, "rl_launch: NULL argument");
+  if (!gx || !gy || !gz || !bx || !by || !bz) return fail(RL_ERR_INVALID_ARG, "rl_launch: empty grid or block");
+  if ((unsigned long)bx * by * bz > 1024) return fail(RL_ERR_INVALID_ARG, "rl_launch: more than 1024 threads per block");
+  for (int i = 0; i < n_args; ++i)
+    if (!args[i]) return fail(RL_ERR_INVALID_ARG, "rl_launch: args[%d] is NULL", i);
+  HIP_TRY(hipModuleLaunchKernel((hipFunction_t)f, gx, gy, gz, bx, by, bz, lds_bytes, (hipStream_t)stream, args, nullptr));
+  return RL_OK;
+}
+
+int rl_malloc(void** dptr, size_t bytes) {
+  if (!dptr) return fail(RL_ERR_INVALID_ARG, "rl_malloc: NULL argument");
+  int rc = ensure_ready();
+  if (rc) return rc;
+  *dptr = nullptr;
+  if (bytes == 0) return RL_OK;
+  HIP_TRY(hipMalloc(dptr, bytes));
+  return RL_OK;
+}
+
+int rl_free(void* dptr) {
+  if (!dptr) return RL_OK;
+  HIP_TRY(hipFree(dptr));
+  return RL_OK;
+}
+
+int rl_memcpy_h2d(void* dst, const void* src, size_t bytes) {
+  if (bytes == 0) return RL_OK;
+  if (!dst || !src) return fail(RL_ERR_INVALID_ARG, "rl_memcpy_h2d: NULL argument");
+  HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  return RL_OK;
+}
+
+int rl_memcpy_d2h(void* dst, const void* src, size_t bytes) {
+  if (bytes == 0) return RL_OK;
+  if (!dst || !src) return fail(RL_ERR_INVALID_ARG, "rl_memcpy_d2h: NULL argument");
+  HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return RL_OK;
+}
+
+int rl_memset(void* dptr, int byte_value, size_t bytes) {
+  if (bytes == 0) return RL_OK;
+  if (!dptr) return fail(RL_ERR_INVALID_ARG, "rl_memset: NULL argument");
+  HIP_TRY(hipMemset(dptr, byte_value, bytes));
+  return RL_OK;
+}
+
+int rl_stream_create(rl_stream* out) {
+  if (!out) return fail(RL_ERR_INVALID_ARG, "rl_stream_create: NULL argument");
+  int rc = ensure_ready();
+  if (rc) return rc;
+  hipStream_t s = nullptr;
+  HIP_TRY(hipStreamCreate(&s));  // default priority on purpose
+  *out = s;
+  return RL_OK;
+}
+
+int rl_stream_destroy(rl_stream s) {
+  if (!s) return RL_OK;
+  HIP_TRY(hipStreamDestroy((hipStream_t)s));
+  return RL_OK;
+}
+
+int rl_event_create(rl_event* out) {
+  if (!out) return fail(RL_ERR_INVALID_ARG, "rl_event_create: NULL argument");
+  int rc = ensure_ready();
+  if (rc) return rc;
+  hipEvent_t e = nullptr;
+  HIP_TRY(hipEventCreate(&e));
+  *out = e;
+  return RL_OK;
+}
+
+int rl_event_record(rl_event e, rl_stream s) {
+  if (!e) return fail(RL_ERR_INVALID_ARG, "rl_event_record: NULL event");
+  HIP_TRY(hipEventRecord((hipEvent_t)e, (hipStream_t)s));
+  return RL_OK;
+}
+
+int rl_event_sync(rl_event e) {
+  if (!e) return fail(RL_ERR_INVALID_ARG, "rl_event_sync: NULL event");
+  HIP_TRY(hipEventSynchronize((hipEvent_t)e));
+  return RL_OK;
+}
+
+int rl_event_elapsed_ms(rl_event start, rl_event stop, float* ms) {
+  if (!start || !stop || !ms) return fail(RL_ERR_INVALID_ARG, "rl_event_elapsed_ms: NULL argument");
+  HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+  return RL_OK;
+}
+
+int rl_event_destroy(rl_event e) {
+  if (!e) return RL_OK;
+  HIP_TRY(hipEventDestroy((hipEvent_t)e));
+  return RL_OK;
+}
+
+int rl_sync(void) {
+  int rc = ensure_ready();
+  if (rc) return rc;
+  HIP_TRY(hipDeviceSynchronize());
+  return RL_OK;
+}
+
+const char* rl_gemm_template_source(void) { return rl_gemm_template_begin; }
+
+int rl_gemm_config_check(const rl_gemm_config* cfg, int* lds_bytes, int* threads) {
+  if (!cfg) return fail(RL_ERR_INVALID_ARG, "cfg is NULL");
+  return check_config(*cfg, lds_bytes, threads);
+}
+
+int rl_set_cache_dir(const char* path) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (!path || !*path) {
+    g_cache_dir.clear();
+    return RL_OK;
+  }
+  struct stat st;
+  if (stat(path, &st) != 0) {
+    if (mkdir(path, 0777) != 0) return fail(RL_ERR_IO, "cannot create cache directory %s", path);
+  } else if (!S_ISDIR(st.st_mode)) {
+    return fail(RL_ERR_IO, "%s is not a directory", path);
+  }
+  g_cache_dir = path;
+  return RL_OK;
+}
+
+int rl_gemm_precompile(const rl_gemm_config* cfg, size_t* code_size) {
+  if (!cfg) return fail(RL_ERR_INVALID_ARG, "cfg is NULL");
+  int rc = check_config(*cfg, nullptr, nullptr);
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lock(g_mutex);
+  if (g_cache_dir.empty()) return fail(RL_ERR_IO, "rl_gemm_precompile needs a cache directory (rl_set_cache_dir)");
+  std::vector<char> code;
+  rc = code_for(*cfg, &code, nullptr);
+  if (rc) return rc;
+  std::vector<char> check;
+  if (!read_file(cache_path(*cfg), &check)) return fail(RL_ERR_IO, "could not store %s", cache_path(*cfg).c_str());
+  if (code_size) *code_size = code.size();
+  return RL_OK;
+}
+
+int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* compile_ms) {
+  if (compile_ms) *compile_ms = 0.0f;
+  if (!cfg || !out) return fail(RL_ERR_INVALID_ARG, "rl_gemm_plan_create: NULL argument");
+  *out = nullptr;
+  int lds = 0, threads = 0;
+  int rc = check_config(*cfg, &lds, &threads);
+  if (rc) return rc;
+  rc = ensure_ready();
+  if (rc) return rc;
+
+  std::lock_guard<std::mutex> lock(g_mutex);
+  const std::string key = config_key(*cfg);
+  auto it = g_plans.find(key);
+  if (it != g_plans.end()) {
+    *out = it->second;
+    return RL_OK;
+  }
+  std::vector<char> code;
+  rc = code_for(*cfg, &code, compile_ms);
+  if (rc) return rc;
+
+  rl_gemm_plan* p = new rl_gemm_plan();
+  p->cfg = *cfg;
+  p->lds_bytes = lds;
+  p->threads = threads;
+  hipError_t e = hipModuleLoadData(&p->module, code.data());
+  if (e == hipSuccess) e = hipModuleGetFunction(&p->func, p->module, "gemm_kernel");
+  if (e == hipSuccess && lds > 64 * 1024 && opt_in_lds(p->func, lds) != RL_OK) e = hipErrorInvalidValue;
+  if (e != hipSuccess) {
+    if (p->module) (void)hipModuleUnload(p->module);
+    delete p;
+    return hip_fail(e, "loading the compiled GEMM kernel");
+  }
+  p->vgprs = metadata_int(code, ".vgpr_count");
+  p->agprs = metadata_int(code, ".agpr_count");
+  p->sgprs = metadata_int(code, ".sgpr_count");
+  const int vs = metadata_int(code, ".vgpr_spill_count"), ss = metadata_int(code, ".sgpr_spill_count");
+  p->spilled = (vs < 0 || ss < 0) ? -1 : vs + ss;
+  p->scratch = metadata_int(code, ".private_segment_fixed_size");
+  g_plans[key] = p;
+  *out = p;
+  return RL_OK;
+}
+
+int rl_gemm_plan_function(const rl_gemm_plan* plan, rl_function* out) {
+  if (!plan || !out) return fail(RL_ERR_INVALID_ARG, "rl_gemm_plan_function: NULL argument");
+  *out = plan->func;
+  return RL_OK;
+}
+
+int rl_gemm_plan_lds_bytes(const rl_gemm_plan* plan) { return plan ? plan->lds_bytes : 0; }
+int rl_gemm_plan_threads(const rl_gemm_plan* plan) { return plan ? plan->threads : 0; }
+
+int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int* sgprs,
+                           int* spilled, int* scratch_bytes) {
+  if (!plan) return fail(RL_ERR_INVALID_ARG, "plan is NULL");
+  if (vgprs) *vgprs = plan->vgprs;
+  if (agprs) *agprs = plan->agprs;
+  if (sgprs) *sgprs = plan->sgprs;
+  if (spilled) *spilled = plan->spilled;
+  if (scratch_bytes) *scratch_bytes = plan->scratch;
+  return RL_OK;
+}
+
+int rl_gemm_plans_clear(void) {
+  std::lock_guard<std::mutex> lock(g_mutex);
+  int rc = RL_OK;
+  for (auto& kv : g_plans) {
+    if (kv.second->module) {
+      hipError_t e = hipModuleUnload(kv.second->module);
+      if (e != hipSuccess) rc = hip_fail(e, "hipModuleUnload");
+    }
+    delete kv.second;
+  }
+  g_plans.clear();
+  return rc;
+}
+
+int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
+                        int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream) {
+  if (!plan) return fail(RL_ERR_INVALID_ARG, "plan is NULL");
+  const rl_gemm_config& c = plan->cfg;
+  if (M < 0 || N < 0 || K < 0) return fail(RL_ERR_INVALID_ARG, "negative dimension (M=%d N=%d K=%d)", M, N, K);
+  if (M == 0 || N == 0) return RL_OK;
+  if (!C || (K > 0 && (!A || !B))) return fail(RL_ERR_INVALID_ARG, "NULL matrix pointer");
+  if (lda < K || ldb < N || ldc < N)
+    return fail(RL_ERR_INVALID_ARG, "leading dimension too small (lda=%d K=%d, ldb=%d ldc=%d N=%d)", lda, K, ldb, ldc, N);
+  if (c.vec == 4) {
+    if (K % 4 || N % 4 || lda % 4 || ldb % 4 || ldc % 4)
+      return fail(RL_ERR_INVALID_ARG, "vec=4 kernel needs K, N, lda, ldb, ldc to be multiples of 4 (K=%d N=%d lda=%d ldb=%d ldc=%d)", K, N, lda, ldb, ldc);
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15)
+      return fail(RL_ERR_INVALID_ARG, "vec=4 kernel needs 16-byte aligned A, B and C");
+  } else if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 3) {
+    return fail(RL_ERR_INVALID_ARG, "A, B and C must be 4-byte aligned");
+  }
+  if (!c.edge && (M % c.bm || N % c.bn || K % c.bk))
+    return fail(RL_ERR_INVALID_ARG, "edge=0 kernel needs bm|M, bn|N, bk|K (tile %dx%dx%d, problem %dx%dx%d)", c.bm, c.bn, c.bk, M, N, K);
+  // In-tile byte offsets are 32-bit inside the kernel; 0x80000000 is reserved as "out of range".
+  const long lim = 0x7fffffffL;
+  if ((long)c.bm * lda * 4 + (long)c.bk * 4 > lim || (long)c.bk * ldb * 4 + (long)c.bn * 4 > lim ||
+      (long)c.bm * ldc * 4 + (long)c.bn * 4 > lim)
+    return fail(RL_ERR_INVALID_ARG, "leading dimension too large for 32-bit in-tile offsets");
+  const long nbm = ((long)M + c.bm - 1) / c.bm, nbn = ((long)N + c.bn - 1) / c.bn;
+  if (nbn > 0x7fffffffL || nbm > 65535 || nbm * nbn > lim)
+    return fail(RL_ERR_INVALID_ARG, "tile grid %ldx%ld too large", nbn, nbm);
+
+  void* args[] = {(void*)&A, (void*)&B, (void*)&C, &M, &N, &K, &lda, &ldb, &ldc};
+  HIP_TRY(hipModuleLaunchKernel(plan->func, (unsigned)nbn, (unsigned)nbm, 1, (unsigned)plan->threads, 1, 1,
+                                (unsigned)plan->lds_bytes, (hipStream_t)stream, args, nullptr));
+  return RL_OK;
+}
+
+int rl_gemm_f32(const rl_gemm_config* cfg, const float* A, const float* B, float* C, int M,
+                int N, int K, int lda, int ldb, int ldc, rl_stream stream) {
+  rl_gemm_plan* plan = nullptr;
+  int rc = rl_gemm_plan_create(cfg, &plan, nullptr);
+  if (rc) return rc;
+  return rl_gemm_plan_launch(plan, A, B, C, M, N, K, lda, ldb, ldc, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,470 @@
+"""ctypes binding of libroller_hip.so -- the only way this package reaches the GPU.
+
+It plays the part that CuPy plays in the reference (``cp.cuda.Module``, ``cp.cuda.Event``,
+``cp.zeros`` ..., /root/reference/src/roller.py:498-534): device buffers, events, module load and
+kernel launch, plus the JIT of the GEMM kernel template.  Every call goes through the C ABI in
+``include/roller_hip.h``; a non-zero status becomes a ``HipError`` carrying the library's text,
+so the per-hint ``try/except Exception`` of the benchmark sweep (benchmark.py:43-58) keeps
+working unchanged.
+
+There is no CPU fallback: if the shared library is missing, ``lib()`` raises.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+from dataclasses import dataclass, fields
+from pathlib import Path
+from typing import Optional, Sequence
+
+import numpy as np
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC_DIR = PKG_DIR / "csrc"
+REPO_ROOT = PKG_DIR.parent
+LIB_PATH = PKG_DIR / "libroller_hip.so"
+DEFAULT_CACHE_DIR = PKG_DIR / "_cache"
+ROCM = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
+
+RL_ERR_INVALID_ARG = -1001
+RL_ERR_COMPILE = -1002
+RL_ERR_IO = -1003
+RL_ERR_NO_DEVICE = -1004
+
+
+class HipError(RuntimeError):
+    """A call into libroller_hip.so failed; ``status`` is its return value."""
+
+    def __init__(self, status: int, text: str):
+        super().__init__(f"[{status}] {text}")
+        self.status = status
+
+
+class DeviceProps(C.Structure):
+    _fields_ = [
+        ("name", C.c_char * 128),
+        ("arch", C.c_char * 64),
+        ("compute_units", C.c_int),
+        ("wavefront_size", C.c_int),
+        ("lds_bytes_per_block", C.c_int),
+        ("regs_per_block", C.c_int),
+        ("l2_bytes", C.c_int),
+        ("clock_khz", C.c_int),
+        ("mem_clock_khz", C.c_int),
+        ("mem_bus_bits", C.c_int),
+        ("total_mem_bytes", C.c_size_t),
+    ]
+
+
+class _GemmConfigC(C.Structure):
+    _fields_ = [(n, C.c_int) for n in (
+        "bm", "bn", "bk", "wm", "wn", "mi", "stages", "pad_a", "pad_b", "vec", "edge", "swz",
+        "group", "accum")]
+
+
+@dataclass(frozen=True)
+class GemmConfig:
+    """Parameters of one instance of the kernel template (``rl_gemm_config``)."""
+
+    bm: int = 128
+    bn: int = 128
+    bk: int = 16
+    wm: int = 64
+    wn: int = 64
+    mi: int = 32
+    stages: int = 2
+    pad_a: int = 4
+    pad_b: int = 0
+    vec: int = 4
+    edge: int = 1
+    swz: int = 3
+    group: int = 8
+    accum: int = 0
+
+    def to_c(self) -> _GemmConfigC:
+        return _GemmConfigC(*(getattr(self, f.name) for f in fields(self)))
+
+    @property
+    def threads(self) -> int:
+        return 64 * (self.bm // self.wm) * (self.bn // self.wn)
+
+    @property
+    def lds_bytes(self) -> int:
+        return self.stages * (self.bm * (self.bk + self.pad_a) + self.bk * (self.bn + self.pad_b)) * 4
+
+    def tag(self) -> str:
+        return (f"b{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_mi{self.mi}_s{self.stages}"
+                f"_p{self.pad_a}.{self.pad_b}_v{self.vec}_e{self.edge}_z{self.swz}.{self.group}"
+                f"_a{self.accum}")
+
+
+# --------------------------------------------------------------------------------------------
+# building and loading the shared library
+# --------------------------------------------------------------------------------------------
+
+def build_library(verbose: bool = False) -> Path:
+    """Compiles csrc/roller_hip.cpp into libroller_hip.so (host code; the kernel template is
+    embedded as text and compiled for gfx950 by hiprtc at run time or by ``precompile``)."""
+    template = CSRC_DIR / "gemm_f32_mfma.hip"
+    cmd = [
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+        "-D__HIP_PLATFORM_AMD__", f"-I{ROCM / 'include'}", f"-I{REPO_ROOT / 'include'}",
+        f'-DRL_TEMPLATE_PATH="{template}"', str(CSRC_DIR / "roller_hip.cpp"),
+        "-o", str(LIB_PATH), f"-L{ROCM / 'lib'}", "-lamdhip64", "-lhiprtc",
+        f"-Wl,-rpath,{ROCM / 'lib'}",
+    ]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.run(cmd, check=True)
+    global _lib
+    _lib = None
+    return LIB_PATH
+
+
+_lib: Optional[C.CDLL] = None
+
+_SIGNATURES = {
+    "rl_init": ([C.c_int], C.c_int),
+    "rl_device_info": ([C.POINTER(DeviceProps)], C.c_int),
+    "rl_last_error": ([], C.c_char_p),
+    "rl_compile": ([C.c_char_p, C.c_char_p, C.POINTER(C.c_char_p), C.c_int, C.POINTER(C.c_void_p),
+                    C.POINTER(C.c_size_t), C.POINTER(C.c_void_p)], C.c_int),
+    "rl_free_host": ([C.c_void_p], None),
+    "rl_module_load": ([C.c_void_p, C.POINTER(C.c_void_p)], C.c_int),
+    "rl_module_get_function": ([C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)], C.c_int),
+    "rl_module_unload": ([C.c_void_p], C.c_int),
+    "rl_func_set_max_dynamic_lds": ([C.c_void_p, C.c_int], C.c_int),
+    "rl_launch": ([C.c_void_p] + [C.c_uint] * 7 + [C.c_void_p, C.POINTER(C.c_void_p), C.c_int], C.c_int),
+    "rl_malloc": ([C.POINTER(C.c_void_p), C.c_size_t], C.c_int),
+    "rl_free": ([C.c_void_p], C.c_int),
+    "rl_memcpy_h2d": ([C.c_void_p, C.c_void_p, C.c_size_t], C.c_int),
+    "rl_memcpy_d2h": ([C.c_void_p, C.c_void_p, C.c_size_t], C.c_int),
+    "rl_memset": ([C.c_void_p, C.c_int, C.c_size_t], C.c_int),
+    "rl_stream_create": ([C.POINTER(C.c_void_p)], C.c_int),
+    "rl_stream_destroy": ([C.c_void_p], C.c_int),
+    "rl_event_create": ([C.POINTER(C.c_void_p)], C.c_int),
+    "rl_event_record": ([C.c_void_p, C.c_void_p], C.c_int),
+    "rl_event_sync": ([C.c_void_p], C.c_int),
+    "rl_event_elapsed_ms": ([C.c_void_p, C.c_void_p, C.POINTER(C.c_float)], C.c_int),
+    "rl_event_destroy": ([C.c_void_p], C.c_int),
+    "rl_sync": ([], C.c_int),
+    "rl_gemm_template_source": ([], C.c_char_p),
+    "rl_gemm_config_check": ([C.POINTER(_GemmConfigC), C.POINTER(C.c_int), C.POINTER(C.c_int)], C.c_int),
+    "rl_set_cache_dir": ([C.c_char_p], C.c_int),
+    "rl_gemm_precompile": ([C.POINTER(_GemmConfigC), C.POINTER(C.c_size_t)], C.c_int),
+    "rl_gemm_plan_create": ([C.POINTER(_GemmConfigC), C.POINTER(C.c_void_p), C.POINTER(C.c_float)], C.c_int),
+    "rl_gemm_plan_function": ([C.c_void_p, C.POINTER(C.c_void_p)], C.c_int),
+    "rl_gemm_plan_lds_bytes": ([C.c_void_p], C.c_int),
+    "rl_gemm_plan_threads": ([C.c_void_p], C.c_int),
+    "rl_gemm_plan_resources": ([C.c_void_p] + [C.POINTER(C.c_int)] * 5, C.c_int),
+    "rl_gemm_plans_clear": ([], C.c_int),
+    "rl_gemm_plan_launch": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p], C.c_int),
+    "rl_gemm_f32": ([C.POINTER(_GemmConfigC), C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p], C.c_int),
+}
+
+EXPORTS = tuple(_SIGNATURES)
+
+
+def lib() -> C.CDLL:
+    """The loaded library.  Raises if it has not been built: there is no other GEMM path."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise HipError(RL_ERR_IO, f"{LIB_PATH} is missing; run __graft_entry__.build() "
+                                      "(or mlir_roller_amd.hip.build_library()) first")
+        handle = C.CDLL(str(LIB_PATH))
+        for name, (argtypes, restype) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = restype
+        _lib = handle
+        cache = os.environ.get("ROLLER_HIP_CACHE", str(DEFAULT_CACHE_DIR))
+        if cache:
+            check(handle.rl_set_cache_dir(cache.encode()))
+    return _lib
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise HipError(status, lib().rl_last_error().decode(errors="replace"))
+
+
+_initialised = False
+
+
+def init(device: int = 0) -> None:
+    """Creates the HIP context on ``device`` (once)."""
+    global _initialised
+    if not _initialised:
+        check(lib().rl_init(device))
+        _initialised = True
+
+
+def device_info() -> DeviceProps:
+    init()
+    props = DeviceProps()
+    check(lib().rl_device_info(C.byref(props)))
+    return props
+
+
+def set_cache_dir(path: Optional[os.PathLike]) -> None:
+    check(lib().rl_set_cache_dir(str(path).encode() if path else None))
+
+
+def synchronize() -> None:
+    check(lib().rl_sync())
+
+
+# --------------------------------------------------------------------------------------------
+# device memory, streams, events
+# --------------------------------------------------------------------------------------------
+
+class DeviceArray:
+    """A row-major fp32 (or any dtype) array in HBM; frees its allocation when collected."""
+
+    def __init__(self, shape: Sequence[int], dtype=np.float32):
+        init()
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = C.c_void_p()
+        check(lib().rl_malloc(C.byref(p), self.nbytes))
+        self.ptr = p.value or 0
+
+    @classmethod
+    def from_host(cls, host: np.ndarray) -> "DeviceArray":
+        host = np.ascontiguousarray(host)
+        out = cls(host.shape, host.dtype)
+        out.set(host)
+        return out
+
+    @classmethod
+    def zeros(cls, shape: Sequence[int], dtype=np.float32) -> "DeviceArray":
+        out = cls(shape, dtype)
+        out.fill_bytes(0)
+        return out
+
+    def set(self, host: np.ndarray) -> None:
+        host = np.ascontiguousarray(host, dtype=self.dtype)
+        if host.nbytes != self.nbytes:
+            raise ValueError(f"host array has {host.nbytes} bytes, device array {self.nbytes}")
+        check(lib().rl_memcpy_h2d(self.ptr, host.ctypes.data, self.nbytes))
+
+    def get(self) -> np.ndarray:
+        out = np.empty(self.shape, dtype=self.dtype)
+        check(lib().rl_memcpy_d2h(out.ctypes.data, self.ptr, self.nbytes))
+        return out
+
+    def fill_bytes(self, value: int) -> None:
+        check(lib().rl_memset(self.ptr, value, self.nbytes))
+
+    def free(self) -> None:
+        if getattr(self, "ptr", 0):
+            lib().rl_free(self.ptr)
+            self.ptr = 0
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Stream:
+    """A HIP stream of default priority."""
+
+    def __init__(self):
+        init()
+        p = C.c_void_p()
+        check(lib().rl_stream_create(C.byref(p)))
+        self.handle = p.value
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None):
+                lib().rl_stream_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def _stream_handle(stream) -> Optional[int]:
+    if stream is None:
+        return None
+    return stream.handle if isinstance(stream, Stream) else int(stream)
+
+
+class Event:
+    """Counterpart of ``cp.cuda.Event`` (roller.py:516-522)."""
+
+    def __init__(self):
+        init()
+        p = C.c_void_p()
+        check(lib().rl_event_create(C.byref(p)))
+        self.handle = p.value
+
+    def record(self, stream=None) -> None:
+        check(lib().rl_event_record(self.handle, _stream_handle(stream)))
+
+    def synchronize(self) -> None:
+        check(lib().rl_event_sync(self.handle))
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None):
+                lib().rl_event_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def get_elapsed_time(start: Event, stop: Event) -> float:
+    """Milliseconds between two recorded events (``cp.cuda.get_elapsed_time``, roller.py:580)."""
+    ms = C.c_float()
+    check(lib().rl_event_elapsed_ms(start.handle, stop.handle, C.byref(ms)))
+    return float(ms.value)
+
+
+# --------------------------------------------------------------------------------------------
+# JIT and launch
+# --------------------------------------------------------------------------------------------
+
+def template_source() -> str:
+    return lib().rl_gemm_template_source().decode()
+
+
+def compile_source(source: str, name: str = "kernel.hip", options: Sequence[str] = ()) -> tuple[bytes, str]:
+    """hiprtc: HIP source -> gfx950 code object.  Returns (code, build log); needs no GPU."""
+    opts = (C.c_char_p * max(len(options), 1))(*[o.encode() for o in options])
+    code, size, log = C.c_void_p(), C.c_size_t(), C.c_void_p()
+    status = lib().rl_compile(source.encode(), name.encode(), opts, len(options), C.byref(code),
+                              C.byref(size), C.byref(log))
+    text = C.string_at(log.value).decode(errors="replace") if log.value else ""
+    if log.value:
+        lib().rl_free_host(log)
+    if status != 0:
+        raise HipError(status, lib().rl_last_error().decode(errors="replace"))
+    blob = C.string_at(code.value, size.value)
+    lib().rl_free_host(code)
+    return blob, text
+
+
+class Module:
+    """Counterpart of ``cp.cuda.Module`` (roller.py:504-506)."""
+
+    def __init__(self, code: bytes):
+        init()
+        self._code = C.create_string_buffer(code, len(code))
+        p = C.c_void_p()
+        check(lib().rl_module_load(self._code, C.byref(p)))
+        self.handle = p.value
+
+    def get_function(self, name: str) -> "Function":
+        p = C.c_void_p()
+        check(lib().rl_module_get_function(self.handle, name.encode(), C.byref(p)))
+        return Function(p.value, owner=self)
+
+    def __del__(self):
+        try:
+            if getattr(self, "handle", None):
+                lib().rl_module_unload(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+def _pack_arg(a):
+    if isinstance(a, DeviceArray):
+        return C.c_void_p(a.ptr)
+    if isinstance(a, (C._SimpleCData,)):
+        return a
+    if isinstance(a, (int, np.integer)):
+        # Pointers arrive as Python ints (``dA.data.ptr`` in the reference); anything that does
+        # not fit an int32 is taken to be an address.
+        v = int(a)
+        return C.c_int(v) if -2**31 <= v < 2**31 else C.c_void_p(v)
+    if isinstance(a, (float, np.floating)):
+        return C.c_float(float(a))
+    raise TypeError(f"cannot pass {type(a).__name__} to a kernel")
+
+
+class Function:
+    """A loaded kernel: ``f(grid, block, args, shared_mem=0, stream=None)`` like
+    ``cp.cuda.Function.__call__`` (roller.py:545-550)."""
+
+    def __init__(self, handle: int, owner=None):
+        self.handle = handle
+        self._owner = owner
+
+    def set_max_dynamic_lds(self, nbytes: int) -> None:
+        check(lib().rl_func_set_max_dynamic_lds(self.handle, int(nbytes)))
+
+    def __call__(self, grid, block, args, shared_mem: int = 0, stream=None) -> None:
+        g = tuple(grid) + (1,) * (3 - len(grid))
+        b = tuple(block) + (1,) * (3 - len(block))
+        packed = [_pack_arg(a) for a in args]
+        argv = (C.c_void_p * max(len(packed), 1))(*[C.cast(C.pointer(p), C.c_void_p) for p in packed])
+        check(lib().rl_launch(self.handle, g[0], g[1], g[2], b[0], b[1], b[2], int(shared_mem),
+                              _stream_handle(stream), argv, len(packed)))
+
+
+def config_check(cfg: GemmConfig) -> tuple[int, int]:
+    """(dynamic LDS bytes, threads per workgroup) of ``cfg``; raises if the template rejects it."""
+    lds, threads = C.c_int(), C.c_int()
+    c = cfg.to_c()
+    check(lib().rl_gemm_config_check(C.byref(c), C.byref(lds), C.byref(threads)))
+    return lds.value, threads.value
+
+
+def precompile(cfg: GemmConfig) -> int:
+    """Compiles ``cfg`` into the on-disk cache without a GPU; returns the code-object size."""
+    size = C.c_size_t()
+    c = cfg.to_c()
+    check(lib().rl_gemm_precompile(C.byref(c), C.byref(size)))
+    return size.value
+
+
+class GemmPlan:
+    """One compiled and loaded instance of the kernel template (``rl_gemm_plan``)."""
+
+    def __init__(self, cfg: GemmConfig):
+        init()
+        self.cfg = cfg
+        p, ms = C.c_void_p(), C.c_float()
+        c = cfg.to_c()
+        check(lib().rl_gemm_plan_create(C.byref(c), C.byref(p), C.byref(ms)))
+        self.handle = p.value
+        self.compile_ms = float(ms.value)
+        self.lds_bytes = lib().rl_gemm_plan_lds_bytes(self.handle)
+        self.threads = lib().rl_gemm_plan_threads(self.handle)
+
+    @property
+    def function(self) -> Function:
+        p = C.c_void_p()
+        check(lib().rl_gemm_plan_function(self.handle, C.byref(p)))
+        return Function(p.value, owner=self)
+
+    def resources(self) -> dict:
+        vals = [C.c_int() for _ in range(5)]
+        check(lib().rl_gemm_plan_resources(self.handle, *[C.byref(v) for v in vals]))
+        return dict(zip(("vgprs", "agprs", "sgprs", "spilled", "scratch_bytes"), (v.value for v in vals)))
+
+    def launch(self, A, B, Cm, M: int, N: int, K: int, lda: Optional[int] = None,
+               ldb: Optional[int] = None, ldc: Optional[int] = None, stream=None) -> None:
+        ptr = lambda x: x.ptr if isinstance(x, DeviceArray) else int(x)
+        check(lib().rl_gemm_plan_launch(self.handle, ptr(A), ptr(B), ptr(Cm), M, N, K,
+                                        K if lda is None else lda, N if ldb is None else ldb,
+                                        N if ldc is None else ldc, _stream_handle(stream)))
+
+
+def gemm_f32(cfg: GemmConfig, A, B, Cm, M: int, N: int, K: int, lda=None, ldb=None, ldc=None,
+             stream=None) -> None:
+    """``rl_gemm_f32``: plan lookup (JIT on first use) + launch in one call."""
+    init()
+    ptr = lambda x: x.ptr if isinstance(x, DeviceArray) else int(x)
+    c = cfg.to_c()
+    check(lib().rl_gemm_f32(C.byref(c), ptr(A), ptr(B), ptr(Cm), M, N, K,
+                            K if lda is None else lda, N if ldb is None else ldb,
+                            N if ldc is None else ldc, _stream_handle(stream)))
