@@ -1,0 +1,276 @@
+"""Headline benchmark: fp32 GEMM TFLOP/s of the Roller-selected HIP kernels over M0..M13 on one
+MI355X, as one JSON line on stdout (everything else goes to stderr).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sweep|M0..M13|cfg4] [--topk 20]
+
+A "step" is one pass over the workload: one launch of the best kernel for every shape in it,
+with A, B and C resident in HBM.  Before the timed region, and reported separately, the Roller
+flow of the reference runs per shape (benchmark.py:28-58 there): policy search, JIT of the
+top-k hints, a short timing of each, best one kept.  The winner per shape is remembered in the
+code-object cache directory so that a second run on the same machine (for example under
+rocprofv3) launches the chosen kernels only.  Each winner is verified against a float32 and a
+float64 host GEMM before it is timed; a kernel outside tolerance is discarded and the next best
+takes its place.
+
+The line also carries
+  roofline      the GEMM kernel against the fp32 MFMA peak: algorithmic FLOPs (2*M*N*K per launch,
+                summed over the launches of a step) over the HIP-event time of the timed region,
+                taken on the stream the kernels run on;
+  cpu_baseline  numpy float32 matmul (its BLAS, all host cores) timed on the same inputs, one
+                pass over the workload; a reported figure, not a target;
+  per_shape     ms, TFLOP/s, % of peak, winning hint and its rank for every shape.
+"""
+
+from __future__ import annotations
+
+import argparse
+import contextlib
+import hashlib
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+import numpy as np  # noqa: E402
+
+PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak: 256 CUs * 256 FLOP/clk * 2.4 GHz
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def blas_threads() -> int:
+    try:
+        from threadpoolctl import threadpool_info
+        counts = [p.get("num_threads", 0) for p in threadpool_info() if p.get("user_api") == "blas"]
+        if counts:
+            return int(max(counts))
+    except Exception:
+        pass
+    return int(os.environ.get("OPENBLAS_NUM_THREADS") or os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="sweep", help="sweep (M0..M13), one of M0..M13, or cfg4 (3000x5000x1536)")
+    ap.add_argument("--topk", type=int, default=20)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--retune", action="store_true", help="ignore remembered winners")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (the GEMM path has no multi-GPU part); got --gpus {args.gpus}",
+              file=sys.stderr)
+        return 2
+
+    from mlir_roller_amd import hip
+    from mlir_roller_amd.analyze import MatmulConfig, get_roller_hints
+    from mlir_roller_amd.arch import MI355X
+    from mlir_roller_amd.benchmark import README_SHAPES
+    from mlir_roller_amd.hip import DeviceArray, Event, GemmConfig, GemmPlan, Stream
+    from mlir_roller_amd.roller import gemm_errors, hint_to_gemm_config, make_inputs
+
+    if args.workload == "sweep":
+        names = [f"M{i}" for i in range(14)]
+        shapes = list(README_SHAPES)
+        workload = "M0-M13: the 14 fp32 GEMM shapes of the reference's table, (M,N,K) in {2048,4096,8192}^3"
+    elif args.workload == "cfg4":
+        names, shapes = ["cfg4"], [(3000, 5000, 1536)]
+        workload = "cfg4: M=3000 N=5000 K=1536, standard-normal entries (ragged tiles)"
+    else:
+        idx = int(args.workload.lstrip("Mm"))
+        names, shapes = [f"M{idx}"], [README_SHAPES[idx]]
+        workload = f"M{idx}: M={shapes[0][0]} N={shapes[0][1]} K={shapes[0][2]}"
+    dist = "normal" if args.workload == "cfg4" else "uniform"
+
+    hip.init(0)
+    props = hip.device_info()
+    arch = MI355X.from_device(props)
+    log(f"[bench] {props.name.decode()} {props.arch.decode()} CUs={props.compute_units} clock={props.clock_khz / 1e6:.2f} GHz")
+
+    cache_dir = Path(os.environ.get("ROLLER_HIP_CACHE", str(hip.DEFAULT_CACHE_DIR)))
+    cache_dir.mkdir(parents=True, exist_ok=True)
+    template_id = hashlib.sha1(hip.template_source().encode()).hexdigest()[:12]
+    tuned_path = cache_dir / f"tuned_{template_id}_top{args.topk}.json"
+    tuned = {}
+    if tuned_path.exists() and not args.retune:
+        try:
+            tuned = json.loads(tuned_path.read_text())
+        except Exception:
+            tuned = {}
+
+    stream = Stream()
+    search_s = compile_s = tune_s = verify_s = 0.0
+    cpu_time = cpu_flops = 0.0
+    cases = []
+
+    def time_plan(plan, bufs, shape, reps, warm):
+        M, N, K = shape
+        for _ in range(warm):
+            plan.launch(bufs[0], bufs[1], bufs[2], M, N, K, stream=stream)
+        e0, e1 = Event(), Event()
+        e0.record(stream)
+        for _ in range(reps):
+            plan.launch(bufs[0], bufs[1], bufs[2], M, N, K, stream=stream)
+        e1.record(stream)
+        e1.synchronize()
+        return hip.get_elapsed_time(e0, e1) / reps
+
+    for name, shape in zip(names, shapes):
+        M, N, K = shape
+        cfg = MatmulConfig(M, N, K, 32)
+        A, B = make_inputs(cfg, args.seed, dist)
+        bufs = (DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray.zeros((M, N)))
+
+        t0 = time.perf_counter()
+        hints = get_roller_hints(cfg, arch, topk=args.topk)
+        search_s += time.perf_counter() - t0
+
+        key = f"{M}x{N}x{K}"
+        ranked = []  # (ms, rank, GemmConfig, hint text)
+        if key in tuned:
+            ent = tuned[key]
+            ranked = [(ent["ms"], ent["rank"], GemmConfig(**ent["config"]), ent["hint"])]
+        else:
+            t0 = time.perf_counter()
+            for rank, hint in enumerate(hints, 1):
+                try:
+                    g = hint_to_gemm_config(cfg, hint, 2)
+                    hip.config_check(g)
+                    plan = GemmPlan(g)
+                    compile_s += plan.compile_ms / 1e3
+                    ms = time_plan(plan, bufs, shape, reps=10, warm=3)
+                    ranked.append((ms, rank, g, repr(hint)))
+                except Exception as e:  # a hint may not fit the device: skip it, like the reference's sweep
+                    log(f"[bench] {name} hint {rank} skipped: {e}")
+            tune_s += time.perf_counter() - t0
+            ranked.sort(key=lambda r: r[0])
+        if not ranked:
+            log(f"[bench] {name}: no usable hint")
+            return 1
+
+        # host results: the float32 GEMM doubles as the CPU baseline sample
+        t0 = time.perf_counter()
+        C32 = A @ B
+        t_host = time.perf_counter() - t0
+        if not args.no_cpu_baseline:
+            t0 = time.perf_counter()
+            C32 = np.matmul(A, B, out=C32)
+            t_host = min(t_host, time.perf_counter() - t0)
+        cpu_time += t_host
+        cpu_flops += 2.0 * M * N * K
+
+        t0 = time.perf_counter()
+        chosen = None
+        for ms, rank, g, text in ranked:
+            plan = GemmPlan(g)
+            bufs[2].fill_bytes(0xFF)
+            plan.launch(bufs[0], bufs[1], bufs[2], M, N, K, stream=stream)
+            hip.synchronize()
+            rep = gemm_errors(bufs[2].get(), A, B, C32)
+            if rep["ok"]:
+                chosen = (ms, rank, g, text, plan, rep)
+                break
+            log(f"[bench] {name} hint {rank} outside tolerance, discarded: {rep}")
+        verify_s += time.perf_counter() - t0
+        if chosen is None:
+            log(f"[bench] {name}: every hint failed verification")
+            return 1
+        ms, rank, g, text, plan, rep = chosen
+        tuned[key] = {"ms": ms, "rank": rank, "config": vars(g), "hint": text}
+        log(f"[bench] {name} {shape}: rank {rank}/{len(hints)} {g.tag()}  {ms:.4f} ms  "
+            f"{2.0 * M * N * K / ms / 1e9:.1f} TFLOP/s  normwise {rep['normwise']:.2e} max_abs {rep['max_abs']:.2e}")
+        cases.append({"name": name, "shape": shape, "plan": plan, "bufs": bufs, "rank": rank, "hints": len(hints),
+                      "cfg": g, "hint": text, "rep": rep, "host_ms": t_host * 1e3})
+        del A, B, C32
+
+    with contextlib.suppress(Exception):
+        tuned_path.write_text(json.dumps(tuned, indent=1))
+
+    # ---- the timed region: W warm-up steps, then exactly K steps between two events -------------
+    def one_step():
+        for c in cases:
+            M, N, K = c["shape"]
+            c["plan"].launch(c["bufs"][0], c["bufs"][1], c["bufs"][2], M, N, K, stream=stream)
+
+    for _ in range(args.warmup):
+        one_step()
+    hip.synchronize()
+    e0, e1 = Event(), Event()
+    wall0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        one_step()
+    e1.record(stream)
+    e1.synchronize()
+    hip.synchronize()
+    wall_ms = (time.perf_counter() - wall0) * 1e3
+    total_ms = hip.get_elapsed_time(e0, e1)
+    ms_per_step = total_ms / max(args.steps, 1)
+
+    # per-shape timing of the winners (outside the headline region)
+    per_shape = []
+    for c in cases:
+        M, N, K = c["shape"]
+        ms = time_plan(c["plan"], c["bufs"], c["shape"], reps=max(args.steps, 5), warm=2)
+        tf = 2.0 * M * N * K / ms / 1e9
+        per_shape.append({"name": c["name"], "M": M, "N": N, "K": K, "ms": round(ms, 5), "tflops": round(tf, 2),
+                          "pct_of_peak": round(100 * tf / PEAK_TFLOPS, 1), "kernel": c["cfg"].tag(),
+                          "hint_rank": c["rank"], "hints": c["hints"],
+                          "normwise_err": c["rep"]["normwise"], "max_abs_err": c["rep"]["max_abs"],
+                          "max_abs_bound": c["rep"]["bound"], "host_ms": round(c["host_ms"], 2)})
+
+    flops_per_step = sum(2.0 * s[0] * s[1] * s[2] for s in shapes)
+    bytes_per_step = sum(4.0 * (s[0] * s[2] + s[2] * s[1] + s[0] * s[1]) for s in shapes)
+    tflops = flops_per_step / (ms_per_step * 1e-3) / 1e12
+    launches = len(cases)
+
+    out = {
+        "metric": "fp32 GEMM TFLOP/s (Roller-selected HIP MFMA kernels) over " + ("M0-M13" if args.workload == "sweep" else names[0]),
+        "value": round(tflops, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": workload, "launches_per_step": launches, "inputs": f"{dist}, seed {args.seed}",
+                   "topk": args.topk, "pipeline_depth": 2},
+        "pct_of_fp32_matrix_peak": round(100 * tflops / PEAK_TFLOPS, 2),
+        "roofline": {
+            "bound": "mfma", "achieved": round(tflops, 3), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tflops / PEAK_TFLOPS, 4), "traffic": None,
+            "kernel": "gemm_kernel", "avg_launch_ms": round(ms_per_step / launches, 5),
+            "flops_per_launch": flops_per_step / launches, "algorithmic_bytes_per_launch": bytes_per_step / launches,
+        },
+        "cpu_baseline": None if args.no_cpu_baseline else {
+            "value": round(cpu_flops / cpu_time / 1e12, 4), "unit": "TFLOP/s", "cores": blas_threads(), "kind": "port",
+            "sample": f"numpy float32 matmul, best of 2, one pass over the same {launches} shape(s) and inputs "
+                      f"({cpu_flops / 1e12:.2f} TFLOP in {cpu_time:.1f} s)",
+        },
+        "wall_ms_per_step": round(wall_ms / max(args.steps, 1), 5),
+        "search_s": round(search_s, 3), "compile_s": round(compile_s, 3), "tune_s": round(tune_s, 3),
+        "verify_s": round(verify_s, 3),
+        "device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units,
+                   "clock_mhz": props.clock_khz // 1000},
+        "per_shape": per_shape,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

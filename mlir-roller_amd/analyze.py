@@ -1,0 +1,428 @@
+"""rTile policy: enumerate, validate, rank and complete tile configurations for one fp32 GEMM.
+
+Host surface of /root/reference/src/analyze.py, kept name for name: ``Shape``, ``MatmulConfig``
+(:27-49), ``read_txn_elems`` / ``write_txn_elems`` (:52-59), ``compute_memory_traffic`` (:62-81),
+``TileDict`` (:84-168), ``Policy`` (:171-381) and ``get_roller_hints`` (:384-387).
+
+On the reference's ``CUDA()`` device model the hints that come out are the reference's, in the
+same order (the golden fixtures under tests/golden pin that).  On a device model that has matrix
+cores (``MI355X()``) three things change, all driven by fields of the device model:
+
+* block tiles and reduce steps are multiples of the MFMA granule, and a ladder of such sizes is
+  offered next to the exact divisors, because ragged tiles are predicated by the kernel;
+* the "thread tile" step assigns a *wave* tile: the block tile is split over wavefronts so that
+  every wave owns a grid of MFMA blocks, and ``thread_tile`` is that wave tile seen per lane
+  (the 64 lanes as an 8x8 grid), which keeps ``block_tile // thread_tile`` = threads per block;
+* candidates are ranked by a roofline estimate of the whole GEMM (``Policy.estimate_seconds``)
+  instead of the reference's per-block traffic times wave count.
+"""
+
+from __future__ import annotations
+
+import itertools
+import math
+from dataclasses import dataclass
+from typing import Iterator, List, Optional
+
+from .arch import CUDA, TileDevice  # noqa: F401  (CUDA re-exported like the reference does)
+from .utils import coalesced_factor, coalesced_tensor_shape, factorize, get_all_factors  # noqa: F401
+
+
+@dataclass
+class Shape:
+    """Extent of one GEMM operand as (spatial, reduce)."""
+
+    S: int
+    R: int
+
+    def to_list(self) -> List[int]:
+        return [self.S, self.R]
+
+
+@dataclass
+class MatmulConfig:
+    """C[M,N] = A[M,K] * B[K,N] with ``el_bits``-wide elements."""
+
+    M: int
+    N: int
+    K: int
+    el_bits: int
+
+    def get_input_shapes(self):
+        # Both operands are described as [spatial, reduce]: for the cost model B counts as
+        # [N, K] although it is stored [K, N].
+        return Shape(S=self.M, R=self.K), Shape(S=self.N, R=self.K)
+
+    def get_output_shape(self):
+        return self.M, self.N
+
+    @property
+    def el_bytes(self) -> int:
+        return (self.el_bits + 7) // 8
+
+    @staticmethod
+    def propagate_inputs(tile: List[int], rstep: int):
+        """Operand tiles needed for one output tile and ``rstep`` reduce elements."""
+        return Shape(S=tile[0], R=rstep), Shape(S=tile[1], R=rstep)
+
+    @staticmethod
+    def propagate_outputs(tile: List[int]):
+        return tile
+
+
+def read_txn_elems(arch: TileDevice, el_bytes: int) -> int:
+    """Elements per read transaction."""
+    return arch.transaction_size[1] // el_bytes
+
+
+def write_txn_elems(arch: TileDevice, el_bytes: int) -> int:
+    """Elements per write transaction."""
+    return arch.transaction_size[0] // el_bytes
+
+
+def compute_memory_traffic(output_tile: List[int], matmul_config: MatmulConfig, arch: TileDevice) -> int:
+    """Bytes one workgroup moves for ``output_tile`` over the whole of K: both operand panels
+    in, the tile out, each rounded up to whole transactions."""
+    eb = matmul_config.el_bytes
+    rte, wte = read_txn_elems(arch, eb), write_txn_elems(arch, eb)
+    panels = MatmulConfig.propagate_inputs(output_tile, matmul_config.K)
+    moved = sum(
+        coalesced_tensor_shape(panel.to_list(), full.to_list(), rte)
+        for panel, full in zip(panels, matmul_config.get_input_shapes())
+    )
+    moved += coalesced_tensor_shape(output_tile, list(matmul_config.get_output_shape()), wte)
+    return moved * eb
+
+
+def _natural_size(nbytes: float) -> str:
+    """1536 -> '1.5 KiB' (binary units, one decimal)."""
+    if abs(nbytes) < 1024:
+        return f"{int(nbytes)} Bytes"
+    value = float(nbytes)
+    for unit in ("KiB", "MiB", "GiB", "TiB", "PiB"):
+        value /= 1024.0
+        if abs(value) < 1024.0 or unit == "PiB":
+            return f"{value:.1f} {unit}"
+    return f"{value:.1f} PiB"
+
+
+class TileDict:
+    """One candidate: the schedule (block tile, thread tile, reduce step) plus what the cost
+    model derived for it.  Attribute names are the reference's; ``wave_tile``, ``mfma`` and
+    ``threads`` are filled on devices with matrix cores."""
+
+    def __init__(self, block_tile: List[int], matmul_config: MatmulConfig, rstep: int) -> None:
+        self.matmul_config = matmul_config
+        # schedule
+        self.block_tile = block_tile
+        self.thread_tile: List[int] = []
+        self.rstep = rstep
+        self.wave_tile: List[int] = []
+        self.mfma = 0
+        self.threads = 0
+        self.lds_row_pad = 0
+        # analysis
+        self.traffic = -1
+        self.smem_cost = -1
+        self.block_per_SM = -1
+        self.num_wave = -1
+        self.grid_size = -1
+        self.valid = True
+
+    def __hash__(self) -> int:
+        return hash(tuple(self.block_tile + self.thread_tile))
+
+    def __repr__(self) -> str:
+        text = (
+            f"TileDict(block_tile={self.block_tile}, thread_tile={self.thread_tile}, "
+            f"rstep={self.rstep}, block traffic={_natural_size(self.traffic)}, "
+            f"total traffic={_natural_size(self.traffic * self.grid_size)}, "
+            f"smem_cost={_natural_size(self.smem_cost)}, block_per_SM={self.block_per_SM}, "
+            f"num_wave={self.num_wave}, grid_size={self.grid_size}"
+        )
+        if self.wave_tile:
+            text += f", wave_tile={self.wave_tile}, mfma={self.mfma}, threads={self.threads}"
+        return text + ")"
+
+    def clone(self) -> "TileDict":
+        twin = TileDict(list(self.block_tile), self.matmul_config, self.rstep)
+        twin.__dict__.update(self.__dict__)
+        twin.block_tile = list(self.block_tile)
+        twin.thread_tile = list(self.thread_tile)
+        twin.wave_tile = list(self.wave_tile)
+        return twin
+
+    def infer_smem_usage(self, rstep: Optional[int] = None) -> int:
+        """Bytes of workgroup memory for one pipeline stage: an [m, rstep] and an [rstep, n] tile."""
+        step = self.rstep if rstep is None else rstep
+        # the kernel pads every row of the [m, rstep] tile by ``lds_row_pad`` elements
+        return (step * sum(self.block_tile) + self.lds_row_pad * self.block_tile[0]) * self.matmul_config.el_bytes
+
+    @classmethod
+    def from_block_tile(cls, block_tile: List[int], rstep: int, matmul_config: MatmulConfig,
+                        arch: TileDevice) -> "TileDict":
+        """Cost model of one block tile.  A tile that overflows workgroup memory or the register
+        file comes back with ``valid = False`` and its analysis fields still at -1."""
+        td = cls(block_tile, matmul_config, rstep)
+        td.lds_row_pad = arch.lds_row_pad
+
+        td.smem_cost = td.infer_smem_usage()
+        if td.smem_cost > arch.smem_cap:
+            td.valid = False
+            return td
+
+        reg_usage = int(2 * math.prod(block_tile) * matmul_config.el_bytes / arch.reg_estimate_divisor)
+        if reg_usage > arch.reg_cap:
+            td.valid = False
+            return td
+
+        td.grid_size = math.prod(-(-full // tile) for tile, full in zip(block_tile, matmul_config.get_output_shape()))
+        td.traffic = compute_memory_traffic(block_tile, matmul_config, arch)
+        td.block_per_SM = min(
+            arch.max_smem_usage // max(td.smem_cost, 1),
+            arch.reg_cap // max(reg_usage, 1),
+            arch.sm_partition,
+        )
+        resident = td.block_per_SM * arch.compute_max_core
+        if resident <= 0:
+            td.valid = False
+            return td
+        td.num_wave = -(-td.grid_size // resident)
+        return td
+
+
+def _similarity(a: float, b: float) -> float:
+    """1 when a == b, falling towards 0 as the ratio a/b moves away from 1."""
+    return (2 * a * b) / (a * a + b * b)
+
+
+def split_block_over_waves(block_tile: List[int], waves: int, rstep: int, arch: TileDevice):
+    """Wave tile ``[wm, wn]`` and MFMA size for a block tile computed by ``waves`` wavefronts,
+    or None.  A wave tile must be a grid of MFMA blocks whose column count the kernel reads
+    with one vector load (1, 2 or a multiple of 4 blocks), and the reduce step must hold whole
+    128-bit fragment reads (4 * wave / mi elements of k).  The larger instruction is preferred;
+    among its wave tiles the most square wins, wider before taller."""
+    m, n = block_tile
+    for shape in arch.mfma_shapes:
+        mi = shape[0]
+        if rstep % (4 * arch.warp_size // mi):
+            continue
+        best = None
+        for rows in get_all_factors(waves):
+            cols = waves // rows
+            if m % rows or n % cols:
+                continue
+            wm, wn = m // rows, n // cols
+            if wm % mi or wn % mi:
+                continue
+            col_blocks = wn // mi
+            if not (col_blocks in (1, 2) or col_blocks % 4 == 0):
+                continue
+            key = (wm + wn, -wn)
+            if best is None or key < best[0]:
+                best = (key, [wm, wn])
+        if best is not None:
+            return best[1], mi
+    return None
+
+
+class Policy:
+    """Roller's default policy: small memory traffic per block, few waves of blocks."""
+
+    # tile sizes offered in addition to the exact divisors of a dimension
+    SIMT_LADDER = (2, 4, 8, 16, 32)
+    MFMA_LADDER = (16, 32, 64, 128, 256, 512)
+
+    def __init__(self, config: MatmulConfig, arch: TileDevice) -> None:
+        self.arch = arch
+        self.matmul_config = config
+
+    # ---- device-model helpers -------------------------------------------------------------
+
+    @property
+    def _granule(self) -> int:
+        """Smallest m/n extent of a matrix instruction (0 on SIMT devices)."""
+        shapes = self.arch.mfma_shapes
+        return min(s[0] for s in shapes) if shapes else 0
+
+    @property
+    def _k_granule(self) -> int:
+        """K extent that one 128-bit fragment read feeds on the smallest-k instruction's wave
+        layout: 4 * (wave / m) for every shape, i.e. 8 for 32x32x2 and 16 for 16x16x4."""
+        shapes = self.arch.mfma_shapes
+        return max(4 * self.arch.warp_size // s[0] for s in shapes) if shapes else 0
+
+    # ---- reduce step ------------------------------------------------------------------------
+
+    def _coalesced_score(self, tile: List[int], rstep: int, mode: str = "sim") -> float:
+        """Larger is better.  "sim": how close the contiguous run of each operand tile is to one
+        read transaction (used to pick the base reduce step).  "raw": the summed run lengths
+        (used when the reduce step is grown)."""
+        tiles = MatmulConfig.propagate_inputs(tile, rstep)
+        fulls = self.matmul_config.get_input_shapes()
+        runs = [coalesced_factor(t.to_list(), f.to_list()) for t, f in zip(tiles, fulls)]
+        if mode == "sim":
+            rte = read_txn_elems(self.arch, self.matmul_config.el_bytes)
+            return sum(_similarity(run, rte) for run in runs)
+        return float(sum(runs))
+
+    def get_reduce_step_candidates(self, rstep: int) -> List[int]:
+        """Step sizes tried along a reduce axis of extent ``rstep``: its divisors (no remainder
+        handling needed), or powers of two when it is a large prime.  With matrix cores only
+        multiples of the instruction's k granule qualify and a ladder of such sizes is added,
+        since the kernel predicates a ragged last step."""
+        steps = get_all_factors(rstep)
+        if len(steps) == 2 and rstep > 64:
+            steps = [1]
+            while steps[-1] * 2 < rstep:
+                steps.append(steps[-1] * 2)
+        kg = self._k_granule
+        if kg:
+            ladder = [s for s in (16, 32, 64, 128) if s % kg == 0]
+            steps = sorted({s for s in steps if s % kg == 0} | set(ladder))
+        return steps
+
+    def _assign_reduce_step(self) -> int:
+        steps = self.get_reduce_step_candidates(self.matmul_config.K)
+        return max(steps, key=lambda s: self._coalesced_score([1, 1], s, "sim"))
+
+    # ---- block tiles ------------------------------------------------------------------------
+
+    def _priority(self, td: TileDict) -> float:
+        """Smaller is better."""
+        if self.arch.has_matrix_cores:
+            return self.estimate_seconds(td)
+        return (td.traffic + 1) * td.num_wave
+
+    def estimate_seconds(self, td: TileDict) -> float:
+        """Roofline estimate of the whole GEMM with block tile ``td`` on a device with matrix
+        cores.  The busiest CU works through ceil(grid / CUs) tiles one after another; a tile
+        costs the larger of its MFMA time at the CU's share of the matrix peak and its traffic
+        at the CU's share of the memory bandwidth, plus a fixed cost for filling the pipeline
+        and draining the accumulators that does not shrink with the tile."""
+        a, cfg = self.arch, self.matmul_config
+        m, n = td.block_tile
+        cu_flops = a.peak_matrix_tflops * 1e12 / a.compute_max_core
+        cu_bw = a.bandwidth[0] * 1e9 / a.compute_max_core
+        # padded work: the kernel runs whole MFMA tiles also where the problem is ragged
+        k_steps = -(-cfg.K // td.rstep)
+        t_mfma = 2.0 * m * n * k_steps * td.rstep / cu_flops
+        t_mem = td.traffic / cu_bw
+        # one reduce step of latency exposed at start-up, and the C tile written at the end
+        t_fixed = 2.0e-6 + m * n * cfg.el_bytes / cu_bw
+        tiles_per_cu = -(-td.grid_size // a.compute_max_core)
+        # small wave tiles re-read their LDS fragments more often per MFMA; charge it mildly
+        reuse_penalty = 1.0 + 8.0 / (m + n)
+        return tiles_per_cu * (max(t_mfma * reuse_penalty, t_mem) + t_fixed)
+
+    def get_block_tiles_candidates(self, init_tile: List[int], rstep: int) -> List[TileDict]:
+        """All valid block tiles, best first (stable with respect to enumeration order:
+        m outer, n inner, ascending)."""
+        granule = self._granule
+        ladder = self.MFMA_LADDER if granule else self.SIMT_LADDER
+        steps = []
+        for lower, extent in zip(init_tile, self.matmul_config.get_output_shape()):
+            sizes = {f for f in get_all_factors(extent) if f >= lower}
+            sizes |= {s for s in ladder if lower < s < extent}
+            if granule:
+                sizes = {s for s in sizes if s % granule == 0} or {granule}
+            steps.append(sorted(sizes))
+
+        tiles = []
+        for m, n in itertools.product(*steps):
+            td = TileDict.from_block_tile([m, n], rstep, self.matmul_config, self.arch)
+            if td.valid:
+                tiles.append(td)
+        return sorted(tiles, key=self._priority)
+
+    def _expand_reduce_axis(self, td: TileDict) -> None:
+        """Grows ``td.rstep`` to the multiple of the base step that gives the longest contiguous
+        operand rows while one stage still fits the block's share of workgroup memory.  Only
+        ``rstep`` and ``smem_cost`` change; occupancy figures keep their base-step values."""
+        limit = min(self.arch.max_smem_usage // td.block_per_SM, self.arch.smem_cap)
+        steps = [
+            s for s in self.get_reduce_step_candidates(self.matmul_config.K)
+            if s % td.rstep == 0 and td.infer_smem_usage(s) <= limit
+        ] or [td.rstep]
+        td.rstep = max(steps, key=lambda s: self._coalesced_score(td.block_tile, s, "raw"))
+        td.smem_cost = td.infer_smem_usage()
+
+    # ---- threads per block --------------------------------------------------------------------
+
+    def score_block_size(self, n: int):
+        """(distance of the warp count from one warp per scheduler, fraction of idle lanes in
+        the last warp); smaller is better."""
+        warp, part = self.arch.warp_size, self.arch.sm_partition
+        warps = -(-n // warp)
+        return (max(warps / part, part / warps), (warps * warp - n) / n)
+
+    def recommend_block_size(self, td: TileDict) -> List[int]:
+        """Thread counts worth trying for ``td``: divisors of the tile area up to 1024, best first."""
+        sizes = [t for t in get_all_factors(math.prod(td.block_tile)) if t <= 1024]
+        return sorted(sizes, key=self.score_block_size)
+
+    def assign_thread_tile(self, td: TileDict, topk: int = 1) -> Iterator[TileDict]:
+        """Yields up to ``topk`` completed copies of ``td``, one per block size in recommended
+        order.  The first block size that cannot be tiled ends the sequence."""
+        for block_size in self.recommend_block_size(td):
+            done = self._assign_thread_tile(td, block_size)
+            if done is None:
+                return
+            yield done
+            topk -= 1
+            if topk == 0:
+                return
+
+    def _assign_thread_tile(self, td: TileDict, block_size: int) -> Optional[TileDict]:
+        if self.arch.has_matrix_cores:
+            return self._assign_wave_tile(td, block_size)
+        area = math.prod(td.block_tile) // block_size
+        pairs = [[area // i, i] for i in range(1, math.isqrt(area) + 1) if area % i == 0]
+        k, lds_bw = self.matmul_config.K, self.arch.bandwidth[1]
+        # operand elements a thread reads per output tile: the most square tile reads least
+        best = min(pairs, key=lambda p: sum(math.prod(s.to_list()) / lds_bw
+                                            for s in MatmulConfig.propagate_inputs(p, k)))
+        if int(math.prod(best) * self.matmul_config.el_bytes / 4) >= self.arch.thread_reg_limit:
+            return None
+        td.thread_tile = best
+        return td.clone()
+
+    def _assign_wave_tile(self, td: TileDict, block_size: int) -> Optional[TileDict]:
+        """The thread-tile step on a device with matrix cores: the block tile is split over
+        ``block_size / wave`` wavefronts (see ``split_block_over_waves``)."""
+        warp = self.arch.warp_size
+        if block_size % warp:
+            return None
+        split = split_block_over_waves(td.block_tile, block_size // warp, td.rstep, self.arch)
+        if split is None:
+            return None
+        wave_tile, mi = split
+        lanes_side = math.isqrt(warp)  # 64 lanes seen as 8 x 8
+        if wave_tile[0] % lanes_side or wave_tile[1] % lanes_side:
+            return None
+        thread_tile = [wave_tile[0] // lanes_side, wave_tile[1] // lanes_side]
+        if int(math.prod(thread_tile) * self.matmul_config.el_bytes / 4) >= self.arch.thread_reg_limit:
+            return None
+        td.thread_tile = thread_tile
+        td.wave_tile = wave_tile
+        td.mfma = mi
+        td.threads = block_size
+        return td.clone()
+
+    # ---- top level ------------------------------------------------------------------------------
+
+    def emit_config(self, topk: int = 10) -> List[TileDict]:
+        rstep = self._assign_reduce_step()
+        hints: List[TileDict] = []
+        for td in self.get_block_tiles_candidates([1, 1], rstep):
+            self._expand_reduce_axis(td)
+            for hint in self.assign_thread_tile(td, 2):
+                hints.append(hint)
+                if len(hints) >= topk:
+                    return hints
+        return hints
+
+
+def get_roller_hints(matmul_config: MatmulConfig, arch: TileDevice, topk: int = 10) -> List[TileDict]:
+    """Top-``topk`` tile configurations for ``matmul_config`` on ``arch``, best first."""
+    return Policy(matmul_config, arch).emit_config(topk)

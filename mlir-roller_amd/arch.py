@@ -1,0 +1,135 @@
+"""Hardware descriptions consumed by the rTile policy.
+
+``TileDevice`` and ``CUDA`` keep the field names and the A100 numbers of
+/root/reference/src/arch.py:9-61, so a policy run on ``CUDA()`` reproduces the reference's
+ranking.  ``MI355X`` is the model this package is built for.  The extra fields at the end of
+``TileDevice`` default to the constants that the reference hard-codes inside its policy
+(src/analyze.py:145, :361), which is what lets one policy serve both devices.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Tuple
+
+
+@dataclass
+class TileDevice:
+    """One accelerator as the policy sees it.  Capacities are per compute core (SM / CU)."""
+
+    reg_cap: int = 0            # 32-bit registers per core
+    smem_cap: int = 0           # workgroup-memory bytes one block may use per pipeline stage
+    compute_max_core: int = 0   # number of cores (SMs / CUs)
+    warp_size: int = 0          # lanes that execute in lockstep
+    sm_partition: int = 0       # schedulers (SIMDs) per core
+    max_smem_usage: int = 0     # workgroup-memory bytes all resident blocks of a core may use
+    platform: str = "unknown"
+    compute_capability: str = "unknown"
+    l2_cache_size_bytes: int = 0
+    # [global write, workgroup-memory read] transaction sizes in bytes
+    transaction_size: List[int] = field(default_factory=lambda: [0, 0])
+    # [device memory, workgroup memory] bandwidth, GB/s
+    bandwidth: List[int] = field(default_factory=lambda: [0, 0])
+
+    # ---- not in the reference's dataclass; defaults = the reference's hard-coded constants ----
+    # a block tile [m, n] is charged int(2*m*n*el_bytes / reg_estimate_divisor) registers
+    reg_estimate_divisor: int = 32
+    # a per-lane accumulator tile needing this many 32-bit registers or more is rejected
+    thread_reg_limit: int = 256
+    # elements of padding the kernel adds to every row of the [m, rstep] workgroup-memory tile
+    lds_row_pad: int = 0
+    # matrix-instruction shapes (m, n, k); empty = no matrix cores modelled, SIMT outer product
+    mfma_shapes: List[Tuple[int, int, int]] = field(default_factory=list)
+    # dies with a private L2 that the dispatcher deals workgroups to round-robin
+    xcd_count: int = 1
+    # dense matrix peak for the dtype of the GEMM, TFLOP/s (0 = unknown)
+    peak_matrix_tflops: float = 0.0
+    # peak engine clock, MHz (0 = unknown)
+    clock_mhz: int = 0
+
+    def get_avaliable_tensorintrin_shapes(self) -> List[Tuple[int, int, int]]:
+        """Matrix-instruction shapes of the device (name kept from the reference, arch.py:36)."""
+        if not self.mfma_shapes:
+            raise NotImplementedError(f"{self.platform} model has no matrix-instruction shapes")
+        return list(self.mfma_shapes)
+
+    @property
+    def has_matrix_cores(self) -> bool:
+        return bool(self.mfma_shapes)
+
+
+@dataclass
+class CUDA(TileDevice):
+    """NVIDIA A100 exactly as the reference models it (arch.py:41-61)."""
+
+    platform: str = "CUDA"
+    reg_cap: int = 65536
+    smem_cap: int = 64 * 1024
+    compute_max_core: int = 108
+    warp_size: int = 32
+    sm_partition: int = 4
+    transaction_size: List[int] = field(default_factory=lambda: [32, 128])
+    bandwidth: List[int] = field(default_factory=lambda: [750, 12080])
+    max_smem_usage: int = field(init=False)
+
+    def __post_init__(self) -> None:
+        self.max_smem_usage = 2 * self.smem_cap
+
+
+@dataclass
+class MI355X(TileDevice):
+    """AMD Instinct MI355X (gfx950, CDNA4).
+
+    256 CUs in 8 XCDs, four SIMDs per CU, 64-lane wavefronts.  Every SIMD holds 512 32-bit
+    registers per lane (256 architectural + 256 accumulation registers), so a CU holds
+    4 * 512 * 64 = 131072.  A CU has 160 KB of LDS and one workgroup may take all of it; the
+    kernel double-buffers its operand tiles, so the budget of one pipeline stage is half of that.
+    fp32 MFMA (v_mfma_f32_32x32x2_f32 / v_mfma_f32_16x16x4_f32) retires 256 FLOP per clock per CU:
+    256 CUs * 256 * 2.4 GHz = 157.3 TFLOP/s.  HBM3E delivers 8 TB/s; the LDS figure is
+    256 CUs * 128 B/clk * 2.4 GHz.
+    """
+
+    platform: str = "ROCm"
+    compute_capability: str = "gfx950"
+    reg_cap: int = 4 * 512 * 64
+    lds_bytes: int = 160 * 1024
+    compute_max_core: int = 256
+    warp_size: int = 64
+    sm_partition: int = 4
+    l2_cache_size_bytes: int = 4 * 1024 * 1024
+    transaction_size: List[int] = field(default_factory=lambda: [64, 128])
+    bandwidth: List[int] = field(default_factory=lambda: [8000, 78643])
+    # accumulators (m*n) plus about as much again for operand fragments and staging registers
+    reg_estimate_divisor: int = 4
+    # 256 accumulation registers per lane are available next to the architectural ones
+    thread_reg_limit: int = 257
+    # rows of the LDS A tile are padded by one 16-byte unit so that 128-bit reads of
+    # consecutive rows fall into distinct bank groups
+    lds_row_pad: int = 4
+    mfma_shapes: List[Tuple[int, int, int]] = field(default_factory=lambda: [(32, 32, 2), (16, 16, 4)])
+    xcd_count: int = 8
+    peak_matrix_tflops: float = 157.3
+    clock_mhz: int = 2400
+    smem_cap: int = field(init=False)
+    max_smem_usage: int = field(init=False)
+
+    def __post_init__(self) -> None:
+        self.smem_cap = self.lds_bytes // 2
+        self.max_smem_usage = self.lds_bytes // 2
+
+    @classmethod
+    def from_device(cls, props) -> "MI355X":
+        """Model with the CU count, clock and LDS size that the runtime reports
+        (``rl_device_info``) in place of the data-sheet values."""
+        model = cls()
+        if getattr(props, "compute_units", 0) > 0:
+            model.compute_max_core = int(props.compute_units)
+        if getattr(props, "lds_bytes_per_block", 0) > 0:
+            model.lds_bytes = int(props.lds_bytes_per_block)
+            model.__post_init__()
+        if getattr(props, "clock_khz", 0) > 0:
+            model.clock_mhz = int(props.clock_khz) // 1000
+        if getattr(props, "l2_bytes", 0) > 0:
+            model.l2_cache_size_bytes = int(props.l2_bytes)
+        model.peak_matrix_tflops = model.compute_max_core * 256 * model.clock_mhz * 1e6 / 1e12
+        return model

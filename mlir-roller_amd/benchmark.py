@@ -1,0 +1,149 @@
+"""Sweep driver: for every (M, N, K) take the top-k Roller hints, compile and time each, keep the
+fastest, and tabulate it next to the host baseline.
+
+Same entry point and flow as /root/reference/src/benchmark.py:10-95 -- ``benchmark(test_shapes,
+topk=20)``, per-shape baseline inside try/except (:19-26), per-hint compile + eval inside
+try/except so that one failing hint never ends the sweep (:41-58), a summary table printed and
+written to ``benchmark_results.csv`` (:89-95).  The table keeps the reference's columns (the
+baseline is numpy's BLAS on the host cores instead of CuPy/cuBLAS, so the two "CuPy" columns
+are named "Host") and adds what an MI355X run is judged by: TFLOP/s, % of the fp32-matrix peak,
+policy-search and JIT time, the rank of the winning hint, and the error measures.
+"""
+
+from __future__ import annotations
+
+import argparse
+import itertools
+import os
+import time
+from pathlib import Path
+from typing import List, Optional, Sequence, Tuple
+
+import pandas as pd
+
+from .analyze import MatmulConfig, get_roller_hints
+from .arch import MI355X, TileDevice
+from .roller import Compiler, run_baseline, run_eval
+
+# The fourteen shapes of the reference's result table, M0..M13 as (M, N, K) (README.md:13-17).
+README_SHAPES: List[Tuple[int, int, int]] = [
+    (2048, 2048, 2048), (2048, 2048, 8192), (2048, 4096, 2048), (2048, 4096, 4096),
+    (2048, 8192, 2048), (2048, 8192, 4096), (2048, 8192, 8192), (4096, 2048, 2048),
+    (4096, 4096, 8192), (4096, 8192, 2048), (4096, 8192, 4096), (8192, 2048, 8192),
+    (8192, 4096, 2048), (8192, 4096, 4096),
+]
+
+
+def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
+              arch: Optional[TileDevice] = None, baseline: bool = True,
+              csv_path: Optional[os.PathLike] = "benchmark_results.csv",
+              dump_path: Optional[os.PathLike] = None, repeat_times: int = 20,
+              distribution: str = "uniform", seed: int = 0) -> pd.DataFrame:
+    arch = arch or MI355X()
+    peak_tflops = arch.peak_matrix_tflops or float("nan")
+    results = []
+
+    for m, n, k in test_shapes:
+        print(f"--- Benchmarking M={m}, N={n}, K={k} ---")
+        config = MatmulConfig(M=m, N=n, K=k, el_bits=32)
+
+        # 1. host baseline
+        baseline_time, baseline_gflops = float("inf"), 0
+        if baseline:
+            print("Running baseline (numpy float32 matmul on the host)...")
+            try:
+                baseline_time, baseline_gflops = run_baseline(config, seed=seed)
+                print(f"Host baseline: {baseline_time:.6f} ms, {baseline_gflops:.6f} GFLOPS")
+            except Exception as e:
+                print(f"Host baseline failed: {e}")
+                baseline_time, baseline_gflops = float("inf"), 0
+
+        # 2. roller hints
+        pipeline_depth = 2
+        print(f"Generating and testing {topk} roller hints...")
+        t0 = time.perf_counter()
+        try:
+            hints = get_roller_hints(config, arch, topk=topk)
+        except Exception as e:
+            print(f"Could not get hints for shape ({m},{n},{k}): {e}")
+            hints = []
+        search_s = time.perf_counter() - t0
+
+        best_time, best_gflops, best_hint, best_rank, best_info = float("inf"), 0, None, -1, {}
+        compile_s, failed = 0.0, 0
+        for i, hint in enumerate(hints):
+            print(f"  Testing hint {i + 1}/{len(hints)}: {hint}")
+            try:
+                func = Compiler(config, hint, pipeline_depth,
+                                dump_path=Path(dump_path) if dump_path else None).compile()
+                compile_s += func.compile_ms / 1e3
+                t, gflops = run_eval(func, pipeline_depth, hint, repeat_times=repeat_times,
+                                     seed=seed, distribution=distribution)
+                if t < best_time:
+                    best_time, best_gflops, best_hint, best_rank = t, gflops, hint, i + 1
+                    best_info = dict(func.last_eval)
+            except Exception as e:
+                # a hint may fail to compile, to fit the device or to pass the numerical check
+                failed += 1
+                print(f"    Hint failed with error: {e}")
+                continue
+
+        if best_hint:
+            print(f"Best roller kernel: {best_time:.6f} ms, {best_gflops:.6f} GFLOPS")
+            print(f"Best hint: {best_hint}")
+        else:
+            print("All roller hints failed.")
+
+        # 3. one row per shape
+        tflops = best_gflops / 1e3
+        results.append({
+            "M": m, "N": n, "K": k,
+            "Host Time (ms)": baseline_time,
+            "Host GFLOPS": baseline_gflops,
+            "Roller Time (ms)": best_time,
+            "Roller GFLOPS": best_gflops,
+            "Speedup vs Host": (baseline_time / best_time
+                                if best_time > 0 and baseline_time != float("inf") else 0),
+            "Best Hint": str(best_hint) if best_hint else "N/A",
+            "Roller TFLOPS": tflops,
+            "% of fp32 matrix peak": 100.0 * tflops / peak_tflops,
+            "Best Hint Rank": best_rank,
+            "Hints Tried": len(hints),
+            "Hints Failed": failed,
+            "Search (s)": search_s,
+            "Compile (s)": compile_s,
+            "Normwise Error": best_info.get("normwise", float("nan")),
+            "Max Abs Error": best_info.get("max_abs", float("nan")),
+            "Max Abs Bound": best_info.get("bound", float("nan")),
+        })
+        print("-" * 50)
+
+    # 4. summary
+    df = pd.DataFrame(results)
+    print("\n--- Benchmark Summary ---")
+    print(df.to_string())
+    if csv_path:
+        df.to_csv(csv_path, index=False)
+        print(f"\nResults saved to {csv_path}")
+    return df
+
+
+def main(argv=None) -> None:
+    ap = argparse.ArgumentParser(description="Roller fp32 GEMM sweep on MI355X")
+    ap.add_argument("--shapes", default="readme", choices=["readme", "full"],
+                    help="readme: M0..M13; full: all 27 products of {2048,4096,8192}")
+    ap.add_argument("--topk", type=int, default=20)
+    ap.add_argument("--no-baseline", action="store_true")
+    ap.add_argument("--csv", default="benchmark_results.csv")
+    ap.add_argument("--dump", default=None, help="directory for kernel source / ISA dumps")
+    args = ap.parse_args(argv)
+    if args.shapes == "full":
+        dims = [2048, 4096, 8192]
+        shapes = list(itertools.product(dims, dims, dims))
+    else:
+        shapes = README_SHAPES
+    benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump)
+
+
+if __name__ == "__main__":
+    main()

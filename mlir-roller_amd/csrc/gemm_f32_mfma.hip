@@ -179,9 +179,10 @@ DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool
 }
 
 // Maps the hardware workgroup id to a tile of C.
-DEV void tile_of_workgroup(int nbm, int nbn, int& tile_m, int& tile_n) {
+DEV bool tile_of_workgroup(int nbm, int nbn, int& tile_m, int& tile_n) {
   int pid = blockIdx.y * gridDim.x + blockIdx.x;
   const int npid = nbm * nbn;
+  if (pid >= npid) return false;  // launch wider than the tile grid
 #if SWZ & 1
   // Workgroups are dealt to the XCDs round-robin; undo that so that XCD x works on one
   // contiguous run of the tile order and its L2 sees neighbouring tiles.
@@ -205,6 +206,7 @@ DEV void tile_of_workgroup(int nbm, int nbn, int& tile_m, int& tile_n) {
   tile_m = pid / nbn;
   tile_n = pid % nbn;
 #endif
+  return true;
 }
 
 extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
@@ -222,8 +224,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 
   const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
   int tile_m, tile_n;
-  tile_of_workgroup(nbm, nbn, tile_m, tile_n);
-  if (tile_m >= nbm || tile_n >= nbn) return;  // launch wider than the tile grid
+  if (!tile_of_workgroup(nbm, nbn, tile_m, tile_n)) return;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   // ---- global -> register staging: per-thread loop-invariant offsets ----

@@ -300,8 +300,8 @@ int rl_device_info(rl_device_props* out) {
   hipDeviceProp_t p;
   HIP_TRY(hipGetDeviceProperties(&p, g_device));
   memset(out, 0, sizeof *out);
-  snprintf(out->name, sizeof out->name, "%s", p.name);
-  snprintf(out->arch, sizeof out->arch, "%s", p.gcnArchName);
+  snprintf(out->name, sizeof out->name, "%.127s", p.name);
+  snprintf(out->arch, sizeof out->arch, "%.63s", p.gcnArchName);
   out->compute_units = p.multiProcessorCount;
   out->wavefront_size = p.warpSize;
   out->lds_bytes_per_block = (int)p.sharedMemPerBlockOptin > 0 ? (int)p.sharedMemPerBlockOptin : (int)p.sharedMemPerBlock;

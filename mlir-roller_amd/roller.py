@@ -1,0 +1,317 @@
+"""Compile, launch and time one Roller hint on MI355X.
+
+Keeps the call surface of /root/reference/src/roller.py -- ``Compiler(config, hint,
+pipeline_depth, dump_path).compile()`` (:345-387), the returned handle's
+``f(grid, block, (ptrA, ptrB, ptrC), shared_mem=)`` (:545-550), ``time_cuda`` (:514-522),
+``run_eval`` (:525-586) and ``run_baseline`` (:589-607) -- and replaces what is behind it:
+instead of building a linalg.matmul plus a transform-dialect schedule, lowering it to PTX and
+loading that with CuPy, the hint selects the parameters of a hand-written gfx950 kernel template
+that libroller_hip.so JIT-compiles with hiprtc, caches, loads and launches.
+"""
+
+from __future__ import annotations
+
+import json
+import shutil
+import subprocess
+import time
+from contextlib import contextmanager
+from pathlib import Path
+from typing import Optional, Tuple
+
+import numpy as np
+
+from . import hip
+from .analyze import MatmulConfig, TileDict, get_roller_hints, split_block_over_waves
+from .arch import MI355X
+from .hip import DeviceArray, Event, GemmConfig, GemmPlan
+from .utils import get_block_dims
+
+KERNEL_NAME = "gemm_kernel"  # the symbol the reference looks up (roller.py:499)
+
+# numerical gates of the GEMM path
+NORMWISE_TOL = 1e-5          # ||C - C32||_F / ||C32||_F against a float32 host GEMM
+ELEMENTWISE_FACTOR = 1e-4    # max|C - C64| <= factor * sqrt(K) * max|A| * max|B| against float64
+
+
+def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: int = 2,
+                        accumulate: bool = False) -> GemmConfig:
+    """Template parameters for one hint.
+
+    block_tile -> BM, BN; rstep -> BK; wave_tile -> WM, WN (derived from the thread count when
+    the hint comes from a device model without matrix cores); pipeline_depth -> LDS buffers
+    (the template has 1 or 2).  Ragged problems switch on predication, and problems whose K, N
+    are not multiples of 4 fall back to dword global accesses.
+    """
+    bm, bn = hint.block_tile
+    bk = hint.rstep
+    if hint.wave_tile:
+        (wm, wn), mi = hint.wave_tile, hint.mfma
+    else:
+        threads = 1
+        for d in get_block_dims(hint.block_tile + [0], hint.thread_tile + [0]):
+            threads *= d
+        if threads % 64:
+            raise ValueError(f"{threads} threads per block is not a whole number of 64-lane waves")
+        split = split_block_over_waves(hint.block_tile, threads // 64, bk, MI355X())
+        if split is None:
+            raise ValueError(f"block tile {hint.block_tile} cannot be split into MFMA wave tiles "
+                             f"for {threads} threads and reduce step {bk}")
+        (wm, wn), mi = split
+    M, N, K = config.M, config.N, config.K
+    # (bk + pad)/4 odd keeps the 128-bit reads of LDS-A free of bank conflicts
+    pad_a = 4 if (bk // 4) % 2 == 0 else 0
+    return GemmConfig(
+        bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi,
+        stages=max(1, min(2, int(pipeline_depth))), pad_a=pad_a, pad_b=0,
+        vec=4 if (K % 4 == 0 and N % 4 == 0) else 1,
+        edge=0 if (M % bm == 0 and N % bn == 0 and K % bk == 0) else 1,
+        swz=3, group=8, accum=1 if accumulate else 0,
+    )
+
+
+class KernelHandle:
+    """What ``Compiler.compile()`` returns: a loaded GEMM kernel that is called like the
+    reference's ``cp.cuda.Function``::
+
+        func(grid_dims, block_dims, (ptrA, ptrB, ptrC), shared_mem=nbytes)
+
+    The three pointers are device addresses (ints or ``DeviceArray``).  The kernel takes the
+    problem size at run time, so the handle appends M, N, K and the leading dimensions of the
+    ``MatmulConfig`` it was compiled for (pass nine arguments to override them).  ``grid_dims``
+    and ``block_dims`` are checked -- the grid must cover ceil(N/bn) x ceil(M/bm) tiles and the
+    block must hold the kernel's thread count -- while the launch itself uses the geometry and
+    the (padded) LDS size of the compiled plan.
+    """
+
+    def __init__(self, plan: GemmPlan, config: MatmulConfig, gemm_config: GemmConfig, hint: TileDict):
+        self.plan = plan
+        self.config = config
+        self.gemm_config = gemm_config
+        self.hint = hint
+        self.compile_ms = plan.compile_ms
+        self.last_eval: dict = {}
+
+    @property
+    def shared_mem_bytes(self) -> int:
+        return self.plan.lds_bytes
+
+    @property
+    def threads(self) -> int:
+        return self.plan.threads
+
+    def grid_dims(self) -> Tuple[int, int]:
+        c, g = self.config, self.gemm_config
+        return (-(-c.N // g.bn), -(-c.M // g.bm))
+
+    def block_dims(self) -> Tuple[int, int]:
+        x, y, _ = get_block_dims(self.hint.block_tile + [0], self.hint.thread_tile + [0])
+        return (x, y) if x * y == self.plan.threads else (self.plan.threads, 1)
+
+    def __call__(self, grid_dims, block_dims, args, shared_mem: int = 0, stream=None) -> None:
+        if len(args) == 3:
+            c = self.config
+            dims = (c.M, c.N, c.K, c.K, c.N, c.N)
+        elif len(args) == 9:
+            dims = tuple(int(v) for v in args[3:])
+        else:
+            raise TypeError("args must be (A, B, C) or (A, B, C, M, N, K, lda, ldb, ldc)")
+        M, N, K, lda, ldb, ldc = dims
+        g = self.gemm_config
+        need = (-(-N // g.bn)) * (-(-M // g.bm))
+        have = 1
+        for d in grid_dims:
+            have *= int(d)
+        if have < need:
+            raise ValueError(f"grid {tuple(grid_dims)} has {have} workgroups, the problem needs {need}")
+        lanes = 1
+        for d in block_dims:
+            lanes *= int(d)
+        if lanes != self.plan.threads:
+            raise ValueError(f"block {tuple(block_dims)} has {lanes} threads, the kernel needs {self.plan.threads}")
+        self.plan.launch(args[0], args[1], args[2], M, N, K, lda, ldb, ldc, stream=stream)
+
+
+class Compiler:
+    """Same constructor and ``compile()`` as the reference's ``Compiler`` (roller.py:345-387).
+
+    ``dump_path`` receives ``kernel.hip`` (template source with the chosen parameters as
+    defines), ``kernel.json`` (parameters and register/LDS usage) and, when ``hipcc`` is on the
+    PATH, ``kernel.s`` (gfx950 assembly) -- the counterparts of the reference's
+    ``transformed.mlir`` / ``llvm.mlir`` / ``kernel.ptx`` dumps.
+    """
+
+    def __init__(self, config: MatmulConfig, hint: TileDict, pipeline_depth: int = 2,
+                 dump_path: Optional[Path] = None, accumulate: bool = False):
+        self.config = config
+        self.hint = hint
+        self.pipeline_depth = pipeline_depth
+        self.dump_path = Path(dump_path) if dump_path else None
+        self.accumulate = accumulate
+
+    def compile(self) -> KernelHandle:
+        gemm_config = hint_to_gemm_config(self.config, self.hint, self.pipeline_depth, self.accumulate)
+        hip.config_check(gemm_config)
+        plan = GemmPlan(gemm_config)
+        handle = KernelHandle(plan, self.config, gemm_config, self.hint)
+        if self.dump_path:
+            self._dump(handle)
+        return handle
+
+    def _dump(self, handle: KernelHandle) -> None:
+        out = self.dump_path
+        out.mkdir(parents=True, exist_ok=True)
+        g = handle.gemm_config
+        defines = {k.upper(): v for k, v in vars(g).items()}
+        header = "".join(f"#define {k} {v}\n" for k, v in defines.items())
+        (out / "kernel.hip").write_text(header + hip.template_source())
+        info = {"config": vars(g), "lds_bytes": handle.shared_mem_bytes, "threads": handle.threads,
+                "resources": handle.plan.resources(), "compile_ms": handle.compile_ms}
+        (out / "kernel.json").write_text(json.dumps(info, indent=1))
+        hipcc = shutil.which("hipcc")
+        if hipcc:
+            subprocess.run([hipcc, "--offload-arch=gfx950", "-O3", "--cuda-device-only", "-S",
+                            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                            str(out / "kernel.hip"), "-o", str(out / "kernel.s")],
+                           check=False, capture_output=True)
+
+
+@contextmanager
+def time_cuda(stream=None):
+    """Event pair around a region (name kept from roller.py:514-522); read the result with
+    ``hip.get_elapsed_time(start, end)`` after the block."""
+    start, end = Event(), Event()
+    start.record(stream)
+    yield start, end
+    end.record(stream)
+    end.synchronize()
+
+
+time_hip = time_cuda
+
+
+def make_inputs(config: MatmulConfig, seed: int = 0, distribution: str = "uniform"):
+    """Seeded row-major fp32 operands: uniform[-1, 1), standard normal, or small integers
+    (0..9, for which every fp32 partial sum is exact and any summation order agrees bitwise)."""
+    rng = np.random.default_rng(seed)
+    shape_a, shape_b = (config.M, config.K), (config.K, config.N)
+    if distribution == "uniform":
+        draw = lambda s: rng.uniform(-1.0, 1.0, s).astype(np.float32)
+    elif distribution == "normal":
+        draw = lambda s: rng.standard_normal(s, dtype=np.float32)
+    elif distribution == "integer":
+        draw = lambda s: rng.integers(0, 10, s).astype(np.float32)
+    else:
+        raise ValueError(f"unknown distribution {distribution!r}")
+    return draw(shape_a), draw(shape_b)
+
+
+def gemm_errors(C: np.ndarray, A: np.ndarray, B: np.ndarray, C32: Optional[np.ndarray] = None) -> dict:
+    """Both error measures of the path and their verdicts: normwise against a float32 host GEMM,
+    elementwise against a float64 host GEMM."""
+    if C32 is None:
+        C32 = A @ B
+    K = A.shape[1]
+    ref_norm = float(np.linalg.norm(C32.astype(np.float64)))
+    normwise = float(np.linalg.norm(C.astype(np.float64) - C32.astype(np.float64))) / max(ref_norm, 1e-300)
+    C64 = A.astype(np.float64) @ B.astype(np.float64)
+    max_abs = float(np.max(np.abs(C.astype(np.float64) - C64))) if C.size else 0.0
+    amax = float(np.max(np.abs(A))) if A.size else 0.0
+    bmax = float(np.max(np.abs(B))) if B.size else 0.0
+    bound = ELEMENTWISE_FACTOR * np.sqrt(max(K, 1)) * amax * bmax
+    return {"normwise": normwise, "max_abs": max_abs, "bound": float(bound),
+            "ok": bool(normwise <= NORMWISE_TOL and max_abs <= bound)}
+
+
+_reference_cache: dict = {}
+
+
+def _host_case(config: MatmulConfig, seed: int, distribution: str):
+    """Inputs and float32 host result for a shape; the last one is kept because a sweep
+    evaluates up to ``topk`` hints on the same shape."""
+    key = (config.M, config.N, config.K, seed, distribution)
+    if key not in _reference_cache:
+        _reference_cache.clear()
+        A, B = make_inputs(config, seed, distribution)
+        _reference_cache[key] = (A, B, A @ B)
+    return _reference_cache[key]
+
+
+def run_eval(cuda_func: KernelHandle, pipeline_depth, hint: TileDict, repeat_times: int = 20,
+             seed: int = 0, distribution: str = "uniform", check: bool = True):
+    """Protocol of the reference's ``run_eval`` (roller.py:525-586): one checked launch, one
+    more single launch, ten warm-ups, then ``repeat_times`` launches between two events.
+    Returns ``(ms_per_launch, gflops)``; details land in ``cuda_func.last_eval``.
+
+    Unlike the reference, which only prints on a mismatch, a result outside the tolerances
+    raises, so that a wrong kernel can never be picked as the fastest one.
+    """
+    cfg = hint.matmul_config
+    M, N, K = cfg.M, cfg.N, cfg.K
+    A, B, C32 = _host_case(cfg, seed, distribution)
+    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B)
+    dC = DeviceArray.zeros((M, N))
+
+    g = cuda_func.gemm_config
+    grid_dims = (-(-N // g.bn), -(-M // g.bm))  # the reference floors here; ragged tiles exist now
+    block_dims = cuda_func.block_dims()
+    shared_memory_usage = max(hint.smem_cost * int(pipeline_depth), cuda_func.shared_mem_bytes)
+    args = (dA.ptr, dB.ptr, dC.ptr)
+
+    cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
+    hip.synchronize()
+    info: dict = {}
+    if check:
+        info = gemm_errors(dC.get(), A, B, C32)
+        if not info["ok"]:
+            raise AssertionError(f"GEMM result outside tolerance for {hint}: {info}")
+
+    cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
+    for _ in range(10):
+        cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
+    with time_cuda() as (start_gpu, end_gpu):
+        for _ in range(repeat_times):
+            cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
+    t_gpu = hip.get_elapsed_time(start_gpu, end_gpu)
+
+    flops = 2 * M * N * K
+    gflops = repeat_times * flops * 1e-9 / (t_gpu / 1000)
+    print(f"t={t_gpu / repeat_times:.6f} ms GFLOPS={gflops:.6f}")
+    info.update(ms=t_gpu / repeat_times, gflops=gflops)
+    cuda_func.last_eval = info
+    return t_gpu / repeat_times, gflops
+
+
+def run_baseline(config: MatmulConfig, repeat_times: int = 3, seed: int = 0):
+    """Baseline column of the sweep.  The reference times cuBLAS through ``cp.matmul``
+    (roller.py:589-607); here it is numpy's float32 ``A @ B`` (its BLAS, all host cores) on the
+    same seeded inputs: one warm-up, then the best of ``repeat_times`` wall-clock runs.
+    Returns ``(ms, gflops)``."""
+    A, B, _ = _host_case(config, seed, "uniform")
+    out = np.empty((config.M, config.N), dtype=np.float32)
+    np.matmul(A, B, out=out)
+    best = float("inf")
+    for _ in range(max(1, repeat_times)):
+        t0 = time.perf_counter()
+        np.matmul(A, B, out=out)
+        best = min(best, time.perf_counter() - t0)
+    gflops = 2 * config.M * config.N * config.K * 1e-9 / best
+    print(f"t={best * 1e3:.6f} ms GFLOPS={gflops:.6f}")
+    return best * 1e3, gflops
+
+
+if __name__ == "__main__":
+    S = 4096
+    config = MatmulConfig(M=S, N=S, K=S, el_bits=32)
+    pipeline_depth = 2
+    hints = get_roller_hints(config, MI355X(), topk=20)
+    run_baseline(config)
+    timings = {}
+    for hint in hints:
+        func = Compiler(config, hint, pipeline_depth, dump_path=Path("log")).compile()
+        print(hint)
+        timings[hint] = run_eval(func, pipeline_depth, hint)
+        print("---\n")
+    if timings:
+        best_hint = min(timings, key=lambda h: timings[h][0])
+        print(f"Best hint: {best_hint}, time: {timings[best_hint][0]}, GFLOPS: {timings[best_hint][1]}")

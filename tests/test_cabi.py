@@ -1,0 +1,123 @@
+"""The C ABI without a device: the library loads, exports every symbol that
+include/roller_hip.h declares, validates its arguments, JIT-compiles for gfx950 (hiprtc needs no
+GPU) and maintains its on-disk code-object cache.  No compute call is made here."""
+
+import ctypes as C
+import re
+from pathlib import Path
+
+import pytest
+
+from mlir_roller_amd import hip
+from mlir_roller_amd.hip import GemmConfig, HipError
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = (ROOT / "include" / "roller_hip.h").read_text()
+
+
+def declared_functions():
+    body = re.sub(r"/\*.*?\*/", "", HEADER, flags=re.S)
+    return sorted(set(re.findall(r"\b(rl_[a-z0-9_]+)\s*\(", body)))
+
+
+def test_every_declared_symbol_is_exported(hip_lib):
+    names = declared_functions()
+    assert len(names) >= 35 and "rl_gemm_f32" in names and "rl_launch" in names
+    for name in names:
+        assert hasattr(hip_lib, name), f"{name} declared in roller_hip.h but not exported"
+    # and the binding knows every one of them (argument types set, nothing bound by accident)
+    assert sorted(hip.EXPORTS) == names
+
+
+def test_every_declaration_cites_the_reference_or_says_why_not():
+    # each block comment in the ABI section names a reference file:line
+    assert HEADER.count("src/roller.py:") >= 10 and "src/arch.py:" in HEADER and "benchmark.py:" in HEADER
+
+
+def test_template_source_is_embedded_verbatim(hip_lib):
+    on_disk = (ROOT / "mlir-roller_amd" / "csrc" / "gemm_f32_mfma.hip").read_text()
+    assert hip.template_source() == on_disk
+    assert 'extern "C" __global__' in on_disk and "gemm_kernel" in on_disk
+
+
+def test_config_check_accepts_and_sizes(hip_lib):
+    lds, threads = hip.config_check(GemmConfig(256, 256, 32, 128, 128, 32, 2, 4, 0, 4, 0))
+    assert threads == 256 and lds == 2 * (256 * 36 + 32 * 256) * 4
+    cfg = GemmConfig(128, 128, 16, 64, 64)
+    assert hip.config_check(cfg) == (cfg.lds_bytes, cfg.threads)
+
+
+@pytest.mark.parametrize("bad,needle", [
+    (dict(mi=8), "mi must be"),
+    (dict(wm=48), "does not divide block tile"),
+    (dict(wm=64, wn=64, bm=64, bn=64, mi=32, bk=12), "bk must be a multiple"),
+    (dict(bm=96, bn=96, wm=96, wn=96), "wn/mi must be 1, 2 or a multiple of 4"),
+    (dict(stages=3), "stages must be"),
+    (dict(vec=2), "vec must be"),
+    (dict(pad_a=2), "pad_a/pad_b"),
+    (dict(bm=512, bn=512, wm=128, wn=128, bk=64), "exceed"),
+    (dict(bm=1024, bn=1024, wm=32, wn=32, bk=8), "threads per workgroup"),
+    (dict(edge=2), "edge and accum"),
+    (dict(mi=16, bk=8), "bk must be a multiple of 16"),
+])
+def test_config_check_rejects(hip_lib, bad, needle):
+    with pytest.raises(HipError) as err:
+        hip.config_check(GemmConfig(**bad))
+    assert err.value.status == hip.RL_ERR_INVALID_ARG and needle in str(err.value)
+
+
+def test_compile_plain_source_without_gpu(hip_lib):
+    code, log = hip.compile_source('extern "C" __global__ void k(float* p) { p[threadIdx.x] = 1.0f; }', "k.hip")
+    assert code[:4] == b"\x7fELF" and len(code) > 1000
+    with pytest.raises(HipError) as err:
+        hip.compile_source('extern "C" __global__ void k(float* p) { p[0] = undefined_symbol; }', "bad.hip")
+    assert err.value.status == hip.RL_ERR_COMPILE and "undefined_symbol" in str(err.value)
+
+
+def test_template_compiles_for_both_mfma_shapes(hip_lib):
+    src = hip.template_source()
+    for mi, bk in ((32, 16), (16, 16)):
+        code, _ = hip.compile_source(src, "gemm.hip", [f"-DMI={mi}", f"-DBK={bk}", "-DEDGE=1"])
+        assert b"gemm_kernel" in code
+    # a configuration the template must refuse at compile time
+    with pytest.raises(HipError) as err:
+        hip.compile_source(src, "gemm.hip", ["-DBM=128", "-DWM=48"])
+    assert "wave tile must divide block tile" in str(err.value)
+
+
+def test_precompile_fills_the_disk_cache(hip_lib, tmp_path):
+    try:
+        hip.set_cache_dir(tmp_path)
+        cfg = GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 1)
+        size = hip.precompile(cfg)
+        files = list(tmp_path.glob("gemm_*.hsaco"))
+        assert len(files) == 1 and files[0].stat().st_size == size
+        stamp = files[0].stat().st_mtime_ns
+        assert hip.precompile(cfg) == size and files[0].stat().st_mtime_ns == stamp   # cache hit: not rewritten
+        hip.precompile(GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 0))
+        assert len(list(tmp_path.glob("gemm_*.hsaco"))) == 2                             # key covers every field
+        hip.set_cache_dir(None)
+        with pytest.raises(HipError) as err:
+            hip.precompile(cfg)
+        assert err.value.status == hip.RL_ERR_IO
+    finally:
+        hip.set_cache_dir(hip.DEFAULT_CACHE_DIR)
+
+
+def test_null_arguments_are_errors_not_crashes(hip_lib):
+    assert hip_lib.rl_gemm_config_check(None, None, None) == hip.RL_ERR_INVALID_ARG
+    assert hip_lib.rl_device_info(None) == hip.RL_ERR_INVALID_ARG
+    assert hip_lib.rl_gemm_plan_launch(None, None, None, None, 1, 1, 1, 1, 1, 1, None) == hip.RL_ERR_INVALID_ARG
+    assert hip_lib.rl_launch(None, 1, 1, 1, 1, 1, 1, 0, None, None, 0) == hip.RL_ERR_INVALID_ARG
+    assert hip_lib.rl_event_record(None, None) == hip.RL_ERR_INVALID_ARG
+    assert b"NULL" in hip_lib.rl_last_error()
+    assert hip_lib.rl_free(None) == 0 and hip_lib.rl_module_unload(None) == 0   # freeing nothing is fine
+    assert hip_lib.rl_gemm_plan_lds_bytes(None) == 0
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(hip, "_lib", None)
+    monkeypatch.setattr(hip, "LIB_PATH", tmp_path / "libroller_hip.so")
+    with pytest.raises(HipError) as err:
+        hip.lib()
+    assert "missing" in str(err.value)

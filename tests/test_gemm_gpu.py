@@ -1,0 +1,283 @@
+"""Parity of the HIP GEMM path with the oracle, on an MI355X, every call through the C ABI of
+libroller_hip.so (ctypes).  Tolerances are the ones the path is specified with:
+
+    normwise     ||C - C32||_F / ||C32||_F <= 1e-5      C32 = float32 host GEMM
+    elementwise  max|C - C64| <= 1e-4 * sqrt(K) * max|A| * max|B|      C64 = float64 host GEMM
+
+plus bit-exact equality wherever the mathematics allows it (integer-valued inputs, structured
+operands, run-to-run determinism)."""
+
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+
+from mlir_roller_amd import hip, roller
+from mlir_roller_amd import benchmark as bm
+from mlir_roller_amd.analyze import MatmulConfig, get_roller_hints
+from mlir_roller_amd.arch import MI355X
+from mlir_roller_amd.hip import DeviceArray, GemmConfig, GemmPlan, HipError
+from oracle import gemm_oracle as go
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def run_gemm(cfg: GemmConfig, A: np.ndarray, B: np.ndarray, c_init=None) -> np.ndarray:
+    M, K = A.shape
+    N = B.shape[1]
+    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B)
+    if c_init is None:
+        dC = DeviceArray((M, N))
+        dC.fill_bytes(0xFF)  # NaN pattern: every element must be overwritten
+    else:
+        dC = DeviceArray.from_host(c_init)
+    GemmPlan(cfg).launch(dA, dB, dC, M, N, K)
+    hip.synchronize()
+    return dC.get()
+
+
+def test_device_is_an_mi355x(device):
+    assert device.arch.decode().startswith("gfx950")
+    assert device.wavefront_size == 64 and device.compute_units >= 128
+    assert device.lds_bytes_per_block >= 64 * 1024
+    arch = MI355X.from_device(device)
+    assert arch.compute_max_core == device.compute_units
+
+
+# (config, shapes): aligned, ragged in every dimension, smaller than one tile, K not a multiple of BK
+CASES = [
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 0), [(256, 384, 128), (128, 128, 16)]),
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1), [(200, 300, 72), (1, 4, 4), (129, 132, 20), (64, 64, 1000)]),
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 1, 1), [(37, 53, 29), (1, 1, 1), (130, 127, 17), (5, 700, 3)]),
+    (GemmConfig(256, 256, 32, 128, 128, 32, 2, 4, 0, 4, 1), [(512, 768, 160), (300, 520, 100), (256, 256, 32)]),
+    (GemmConfig(256, 256, 16, 128, 128, 32, 2, 4, 0, 4, 0), [(512, 512, 64)]),
+    (GemmConfig(256, 128, 32, 64, 128, 32, 2, 4, 0, 4, 1), [(300, 260, 100)]),
+    (GemmConfig(128, 256, 32, 64, 64, 32, 2, 4, 0, 4, 1), [(300, 260, 100)]),         # 8 waves
+    (GemmConfig(128, 128, 16, 64, 64, 16, 2, 4, 0, 4, 1), [(200, 300, 80), (33, 36, 16)]),  # 16x16x4 MFMA
+    (GemmConfig(64, 64, 16, 16, 64, 16, 2, 4, 0, 1, 1), [(70, 90, 50)]),
+    (GemmConfig(128, 128, 32, 64, 32, 32, 1, 4, 0, 4, 1), [(200, 300, 72)]),           # single LDS buffer, 1 column block
+    (GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 1), [(200, 300, 72)]),
+    (GemmConfig(64, 256, 32, 64, 64, 32, 2, 4, 0, 4, 1), [(100, 600, 96)]),
+    (GemmConfig(32, 512, 32, 32, 128, 32, 2, 4, 0, 4, 1), [(100, 600, 96)]),
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1, 0, 8), [(400, 500, 48)]),     # no workgroup remap
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1, 2, 3), [(1300, 500, 48)]),    # panel walk, ragged panel
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 0, 0, 4, 1), [(200, 300, 72)]),           # unpadded LDS
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 4, 4, 1), [(200, 300, 72)]),           # padded LDS-B
+]
+FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
+
+
+@pytest.mark.parametrize("cfg,shape", FLAT, ids=[f"{c.tag()}-{s[0]}x{s[1]}x{s[2]}" for c, s in FLAT])
+def test_matches_oracle_within_tolerance_and_exactly_on_integers(device, cfg, shape):
+    M, N, K = shape
+    say("case", cfg.tag(), shape)
+    A, B = go.make_inputs(M, N, K, seed=M + 7 * N + 13 * K)
+    got = run_gemm(cfg, A, B)
+    rep = go.error_report(got, A, B, C64=go.c_gemm_f64(A, B))
+    assert rep["ok"], rep
+    Ai, Bi = go.make_inputs(M, N, K, seed=1, distribution="integer")
+    assert np.array_equal(run_gemm(cfg, Ai, Bi), go.c_gemm_f32(Ai, Bi))
+
+
+def test_structured_operands_are_exact(device):
+    cfg = GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1)
+    n = 200
+    B = np.random.default_rng(3).standard_normal((n, 264), dtype=np.float32)
+    assert np.array_equal(run_gemm(cfg, np.eye(n, dtype=np.float32), B), B)                 # I * B = B
+    A = np.random.default_rng(4).standard_normal((136, n), dtype=np.float32)
+    assert np.array_equal(run_gemm(cfg, A, np.eye(n, dtype=np.float32)), A)                 # A * I = A
+    ones = run_gemm(cfg, np.ones((130, 1000), np.float32), np.ones((1000, 140), np.float32))
+    assert np.all(ones == 1000.0)
+    # one-hot A picks single rows of B: catches any transposition or row/column permutation
+    pick = np.zeros((150, n), np.float32)
+    rows = np.random.default_rng(5).integers(0, n, 150)
+    pick[np.arange(150), rows] = 1
+    assert np.array_equal(run_gemm(cfg, pick, B), B[rows])
+
+
+def test_accumulate_mode_adds_into_c(device):
+    M, N, K = 300, 260, 100
+    A, B = go.make_inputs(M, N, K, seed=11, distribution="integer")
+    C0 = np.random.default_rng(12).integers(-50, 50, (M, N)).astype(np.float32)
+    for cfg in (GemmConfig(256, 128, 32, 64, 128, 32, 2, 4, 0, 4, 1, 3, 8, 1),
+                GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 1, 1, 3, 8, 1),
+                GemmConfig(128, 128, 16, 64, 32, 32, 2, 4, 0, 4, 1, 3, 8, 1)):
+        got = run_gemm(cfg, A, B, c_init=C0)
+        assert np.array_equal(got, go.c_gemm_f32(A, B, out=C0.copy(), accumulate=True)), cfg.tag()
+
+
+def test_leading_dimensions_wider_than_the_matrix(device):
+    M, N, K, lda, ldb, ldc = 200, 300, 72, 96, 320, 304
+    rng = np.random.default_rng(21)
+    hA = rng.integers(0, 10, (M, lda)).astype(np.float32)
+    hB = rng.integers(0, 10, (K, ldb)).astype(np.float32)
+    hC = np.full((M, ldc), -7.0, np.float32)
+    dA, dB, dC = DeviceArray.from_host(hA), DeviceArray.from_host(hB), DeviceArray.from_host(hC)
+    GemmPlan(GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1)).launch(dA, dB, dC, M, N, K, lda, ldb, ldc)
+    hip.synchronize()
+    out = dC.get()
+    assert np.array_equal(out[:, :N], go.c_gemm_f32(hA[:, :K], hB[:, :N]))
+    assert np.all(out[:, N:] == -7.0)                               # padding columns untouched
+
+
+def test_empty_and_zero_k(device):
+    plan = GemmPlan(GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1))
+    dC = DeviceArray.from_host(np.full((8, 12), 3.0, np.float32))
+    plan.launch(0, 0, dC, 8, 12, 0)                                 # K = 0: C = 0
+    hip.synchronize()
+    assert np.all(dC.get() == 0.0)
+    dC.set(np.full((8, 12), 3.0, np.float32))
+    plan.launch(0, 0, dC, 0, 12, 4)                                 # M = 0: nothing to do
+    plan.launch(0, 0, dC, 8, 0, 4, ldb=4, ldc=12)
+    hip.synchronize()
+    assert np.all(dC.get() == 3.0)
+
+
+def test_launch_rejects_what_the_kernel_was_not_built_for(device):
+    dA, dB, dC = DeviceArray((256, 256)), DeviceArray((256, 256)), DeviceArray((256, 256))
+    vec4 = GemmPlan(GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1))
+    aligned = GemmPlan(GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 0))
+    for plan, args, needle in [
+        (vec4, (dA, dB, dC, 100, 101, 64), "multiples of 4"),
+        (vec4, (dA, dB, dC, 100, 100, 62), "multiples of 4"),
+        (vec4, (dA.ptr + 4, dB, dC, 100, 100, 64), "16-byte aligned"),
+        (vec4, (dA, dB, dC, 100, 100, 64, 32), "leading dimension too small"),
+        (vec4, (dA, dB, dC, -1, 100, 64), "negative dimension"),
+        (vec4, (0, dB, dC, 100, 100, 64), "NULL matrix pointer"),
+        (aligned, (dA, dB, dC, 200, 256, 64), "edge=0 kernel needs"),
+        (aligned, (dA, dB, dC, 256, 256, 24), "edge=0 kernel needs"),
+    ]:
+        with pytest.raises(HipError) as err:
+            plan.launch(*args)
+        assert err.value.status == hip.RL_ERR_INVALID_ARG and needle in str(err.value)
+    hip.synchronize()
+
+
+def test_results_are_bitwise_reproducible_and_independent_of_tile_order(device):
+    M, N, K = 1024, 1280, 512
+    A, B = go.make_inputs(M, N, K, seed=31)
+    base = GemmConfig(128, 128, 32, 64, 64, 32, 2, 4, 0, 4, 0)
+    first = run_gemm(base, A, B)
+    assert np.array_equal(first, run_gemm(base, A, B))
+    for swz, group in ((0, 8), (1, 8), (2, 4)):
+        other = GemmConfig(128, 128, 32, 64, 64, 32, 2, 4, 0, 4, 0, swz, group)
+        assert np.array_equal(first, run_gemm(other, A, B)), (swz, group)
+    # predication does not change the arithmetic of full tiles either
+    assert np.array_equal(first, run_gemm(GemmConfig(128, 128, 32, 64, 64, 32, 2, 4, 0, 4, 1), A, B))
+
+
+def test_plan_cache_and_one_shot_entry_point(device):
+    cfg = GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 1)
+    p1, p2 = GemmPlan(cfg), GemmPlan(cfg)
+    assert p1.handle == p2.handle and p2.compile_ms == 0.0
+    res = p1.resources()
+    assert res["spilled"] == 0 and res["scratch_bytes"] == 0 and 0 < res["vgprs"] <= 512
+    A, B = go.make_inputs(70, 80, 48, seed=2, distribution="integer")
+    dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray((70, 80))
+    hip.gemm_f32(cfg, dA, dB, dC, 70, 80, 48)                        # rl_gemm_f32
+    hip.synchronize()
+    assert np.array_equal(dC.get(), go.c_gemm_f32(A, B))
+
+
+def test_low_level_module_api_like_the_reference_uses_cupy(device):
+    src = r'''extern "C" __global__ void axpy(float a, const float* x, float* y, int n) {
+        int i = blockIdx.x * blockDim.x + threadIdx.x;
+        if (i < n) y[i] = a * x[i] + y[i];
+    }'''
+    code, _ = hip.compile_source(src, "axpy.hip")
+    func = hip.Module(code).get_function("axpy")
+    x = np.arange(1000, dtype=np.float32)
+    dx, dy = DeviceArray.from_host(x), DeviceArray.from_host(np.ones(1000, np.float32))
+    stream = hip.Stream()
+    start, stop = hip.Event(), hip.Event()
+    start.record(stream)
+    func((4,), (256,), (C.c_float(2.0), dx, dy, 1000), shared_mem=0, stream=stream)
+    stop.record(stream)
+    stop.synchronize()
+    assert hip.get_elapsed_time(start, stop) >= 0.0
+    assert np.array_equal(dy.get(), 2 * x + 1)
+    with pytest.raises(HipError):
+        hip.Module(code).get_function("no_such_kernel")
+    hip.synchronize()
+
+
+# ---- the named configurations at full size -------------------------------------------------------
+
+FULL = [
+    ("cfg1", (2048, 2048, 2048), "uniform"),
+    ("cfg2", (2048, 2048, 8192), "uniform"),
+    ("cfg3", (4096, 8192, 4096), "uniform"),
+    ("cfg4", (3000, 5000, 1536), "normal"),
+]
+
+
+@pytest.mark.parametrize("name,shape,dist", FULL, ids=[f[0] for f in FULL])
+def test_named_configs_full_size_through_policy_and_compiler(device, name, shape, dist, tmp_path):
+    cfg = MatmulConfig(*shape, 32)
+    hints = get_roller_hints(cfg, MI355X.from_device(device), topk=3)
+    A, B = go.make_inputs(*shape, seed=0, distribution=dist)
+    C32, C64 = go.gemm_f32(A, B), go.gemm_f64(A, B)
+    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B)
+    for hint in hints:
+        say(name, hint)
+        func = roller.Compiler(cfg, hint, 2, dump_path=tmp_path if hint is hints[0] else None).compile()
+        dC = DeviceArray((shape[0], shape[1]))
+        dC.fill_bytes(0xFF)
+        func(func.grid_dims(), func.block_dims(), (dA.ptr, dB.ptr, dC.ptr), shared_mem=hint.smem_cost * 2)
+        hip.synchronize()
+        got = dC.get()
+        rep = go.error_report(got, A, B, C32=C32, C64=C64)
+        assert rep["ok"], (hint, rep)
+        func(func.grid_dims(), func.block_dims(), (dA.ptr, dB.ptr, dC.ptr), shared_mem=0)
+        hip.synchronize()
+        assert np.array_equal(got, dC.get())                         # bit-for-bit across runs
+    assert (tmp_path / "kernel.hip").exists() and (tmp_path / "kernel.json").exists()
+
+
+def test_m0_to_m13_exact_on_integer_inputs_at_full_size(device):
+    """Size-independent property: with inputs in {0..9} every partial sum is an integer below
+    2^24, so any correct summation order gives the same float32 bits as the host GEMM."""
+    arch = MI355X.from_device(device)
+    for i, shape in enumerate(bm.README_SHAPES):
+        cfg = MatmulConfig(*shape, 32)
+        hint = get_roller_hints(cfg, arch, topk=1)[0]
+        say(f"M{i}", shape, hint.block_tile, hint.wave_tile, hint.rstep)
+        A, B = go.make_inputs(*shape, seed=i, distribution="integer")
+        func = roller.Compiler(cfg, hint).compile()
+        dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray((shape[0], shape[1]))
+        func(func.grid_dims(), func.block_dims(), (dA, dB, dC))
+        hip.synchronize()
+        assert np.array_equal(dC.get(), go.gemm_f32(A, B)), shape
+
+
+def test_handle_checks_grid_and_block(device):
+    cfg = MatmulConfig(512, 512, 128, 32)
+    hint = get_roller_hints(cfg, MI355X(), topk=1)[0]
+    func = roller.Compiler(cfg, hint).compile()
+    d = DeviceArray((512, 512))
+    gx, gy = func.grid_dims()
+    with pytest.raises(ValueError):
+        func((max(gx - 1, 0) or 1, 1), func.block_dims(), (d, d, d))   # the reference's floor-div grid would miss tiles
+    with pytest.raises(ValueError):
+        func((gx, gy), (32, 1), (d, d, d))
+    with pytest.raises(TypeError):
+        func((gx, gy), func.block_dims(), (d, d))
+
+
+def test_run_eval_and_sweep_end_to_end(device, tmp_path, capsys):
+    cfg = MatmulConfig(1024, 1024, 512, 32)
+    hint = get_roller_hints(cfg, MI355X.from_device(device), topk=1)[0]
+    func = roller.Compiler(cfg, hint, 2).compile()
+    ms, gflops = roller.run_eval(func, 2, hint, repeat_times=5)
+    assert ms > 0 and gflops == pytest.approx(2 * 1024 * 1024 * 512 * 1e-9 / (ms / 1e3), rel=1e-6)
+    assert func.last_eval["ok"] and func.last_eval["normwise"] <= 1e-5
+    df = bm.benchmark([(512, 768, 256), (300, 500, 96)], topk=4, csv_path=tmp_path / "r.csv", repeat_times=3)
+    assert len(df) == 2 and (tmp_path / "r.csv").exists()
+    assert all(df["Best Hint"] != "N/A") and all(df["Normwise Error"] <= 1e-5)
+    assert all(df["Max Abs Error"] <= df["Max Abs Bound"])

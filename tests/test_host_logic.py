@@ -1,0 +1,128 @@
+"""Host logic that needs no device: hint -> template parameters, the error measures, and the
+sweep's failure handling (a hint that fails to compile or to verify is skipped and the best of
+the rest is still reported, as in the reference's benchmark.py:41-58)."""
+
+import numpy as np
+import pytest
+
+from mlir_roller_amd import benchmark as bm
+from mlir_roller_amd import roller
+from mlir_roller_amd.analyze import MatmulConfig, get_roller_hints
+from mlir_roller_amd.arch import CUDA, MI355X
+from mlir_roller_amd.hip import GemmConfig
+
+
+def test_hint_to_gemm_config_aligned_problem():
+    cfg = MatmulConfig(4096, 8192, 4096, 32)
+    hint = next(h for h in get_roller_hints(cfg, MI355X(), 20) if h.block_tile == [256, 256])
+    g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=2)
+    assert (g.bm, g.bn, g.bk, g.wm, g.wn, g.mi) == (256, 256, hint.rstep, 128, 128, 32)
+    assert (g.stages, g.vec, g.edge, g.accum) == (2, 4, 0, 0)
+    assert ((g.bk + g.pad_a) // 4) % 2 == 1          # odd number of 16-byte units per LDS-A row
+    assert g.threads == hint.threads and g.lds_bytes <= 160 * 1024
+    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=1).stages == 1
+    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=5).stages == 2
+    assert roller.hint_to_gemm_config(cfg, hint, accumulate=True).accum == 1
+
+
+def test_hint_to_gemm_config_ragged_problem():
+    cfg = MatmulConfig(3000, 5000, 1536, 32)
+    g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0])
+    assert g.edge == 1 and g.vec == 4                # 5000 and 1536 are multiples of 4
+    cfg = MatmulConfig(37, 53, 29, 32)
+    g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0])
+    assert g.edge == 1 and g.vec == 1
+
+
+def test_hint_from_the_a100_model_still_maps_to_wave_tiles():
+    cfg = MatmulConfig(2048, 2048, 2048, 32)
+    hint = get_roller_hints(cfg, CUDA(), 1)[0]        # [128,128] / [16,8]: 128 threads = 2 waves
+    g = roller.hint_to_gemm_config(cfg, hint)
+    assert (g.bm, g.bn, g.wm, g.wn, g.threads) == (128, 128, 64, 128, 128)
+    bad = hint.clone()
+    bad.thread_tile = [128, 128]                      # one thread: not a whole wave
+    with pytest.raises(ValueError):
+        roller.hint_to_gemm_config(cfg, bad)
+
+
+def test_gemm_errors_verdicts():
+    cfg = MatmulConfig(48, 40, 64, 32)
+    A, B = roller.make_inputs(cfg, seed=1)
+    good = A @ B
+    assert roller.gemm_errors(good, A, B)["ok"]
+    bad = good.copy()
+    bad[0, 0] += 0.5
+    rep = roller.gemm_errors(bad, A, B)
+    assert not rep["ok"] and rep["max_abs"] > rep["bound"]
+    assert rep["bound"] == pytest.approx(1e-4 * 8 * float(np.abs(A).max()) * float(np.abs(B).max()))
+    An, _ = roller.make_inputs(cfg, seed=1, distribution="normal")
+    assert An.dtype == np.float32 and abs(float(An.mean())) < 0.2
+    with pytest.raises(ValueError):
+        roller.make_inputs(cfg, distribution="cauchy")
+
+
+def test_run_baseline_formula(capsys):
+    ms, gflops = roller.run_baseline(MatmulConfig(64, 64, 64, 32), repeat_times=2)
+    assert ms > 0 and gflops == pytest.approx(2 * 64**3 * 1e-9 / (ms / 1e3), rel=1e-9)
+    assert "GFLOPS=" in capsys.readouterr().out
+
+
+class _FakeFunc:
+    compile_ms = 5.0
+
+    def __init__(self, hint):
+        self.hint = hint
+        self.last_eval = {"normwise": 1e-7, "max_abs": 1e-6, "bound": 1e-3}
+
+
+def test_sweep_survives_failing_hints(monkeypatch, tmp_path):
+    calls = {"compiled": 0}
+
+    class FakeCompiler:
+        def __init__(self, config, hint, depth, dump_path=None):
+            self.hint = hint
+
+        def compile(self):
+            calls["compiled"] += 1
+            if calls["compiled"] % 3 == 1:
+                raise RuntimeError("hiprtc says no")
+            return _FakeFunc(self.hint)
+
+    def fake_eval(func, depth, hint, repeat_times=20, seed=0, distribution="uniform"):
+        if hint.block_tile == [128, 128]:
+            raise AssertionError("result outside tolerance")
+        ms = 1.0 + 0.01 * hint.block_tile[0]
+        return ms, 2 * hint.matmul_config.M * hint.matmul_config.N * hint.matmul_config.K * 1e-9 / (ms / 1e3)
+
+    monkeypatch.setattr(bm, "Compiler", FakeCompiler)
+    monkeypatch.setattr(bm, "run_eval", fake_eval)
+    monkeypatch.setattr(bm, "run_baseline", lambda config, seed=0: (_ for _ in ()).throw(MemoryError("host")))
+    csv = tmp_path / "out.csv"
+    df = bm.benchmark([(2048, 2048, 2048), (4096, 8192, 4096)], topk=6, csv_path=csv)
+    assert len(df) == 2 and csv.exists()
+    r = df.iloc[0]
+    assert r["Hints Tried"] == 6 and r["Hints Failed"] >= 2
+    assert r["Host Time (ms)"] == float("inf") and r["Host GFLOPS"] == 0 and r["Speedup vs Host"] == 0
+    assert r["Roller Time (ms)"] < float("inf") and r["Best Hint"] != "N/A" and r["Best Hint Rank"] >= 1
+    assert r["% of fp32 matrix peak"] == pytest.approx(100 * r["Roller TFLOPS"] / 157.3, rel=1e-3)
+    for col in ("M", "N", "K", "Roller Time (ms)", "Roller GFLOPS", "Best Hint"):   # the reference's columns
+        assert col in df.columns
+
+
+def test_sweep_reports_all_failed(monkeypatch):
+    class AlwaysFails:
+        def __init__(self, *a, **k):
+            pass
+
+        def compile(self):
+            raise RuntimeError("nope")
+
+    monkeypatch.setattr(bm, "Compiler", AlwaysFails)
+    df = bm.benchmark([(2048, 2048, 2048)], topk=3, baseline=False, csv_path=None)
+    assert df.iloc[0]["Best Hint"] == "N/A" and df.iloc[0]["Roller GFLOPS"] == 0
+
+
+def test_readme_shapes_are_the_fourteen():
+    assert len(bm.README_SHAPES) == 14 and bm.README_SHAPES[0] == (2048, 2048, 2048)
+    assert bm.README_SHAPES[10] == (4096, 8192, 4096) and bm.README_SHAPES[13] == (8192, 4096, 4096)
+    assert all(d in (2048, 4096, 8192) for s in bm.README_SHAPES for d in s)

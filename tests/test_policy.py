@@ -1,0 +1,276 @@
+"""Host policy: mlir_roller_amd.{utils,arch,analyze}.
+
+Three layers of evidence that the product policy means what the reference's means:
+  1. golden vectors written by the reference's own code on its A100 model
+     (tests/golden/policy_a100.json): complete ordered top-20 hint lists for M0..M13 and six more
+     shapes, ranked block tiles, block-size orders, and the integer helpers;
+  2. known answers derived by hand from the reference's source (closed forms, first hint);
+  3. an independent plain restatement (oracle/policy_oracle.py), itself pinned by (1), compared
+     with the product on shapes the fixture does not hold.
+Then the MI355X model: MFMA-aligned tiles, wave tiles, resource limits, ranking sanity.
+"""
+
+import itertools
+import math
+import random
+
+import pytest
+
+from mlir_roller_amd import analyze, utils
+from mlir_roller_amd.analyze import MatmulConfig, Policy, TileDict, get_roller_hints
+from mlir_roller_amd.arch import CUDA, MI355X, TileDevice
+from mlir_roller_amd.roller import hint_to_gemm_config
+from oracle import policy_oracle as po
+
+
+def row(td):
+    thread = list(td.thread_tile) or [0, 0]
+    return [*td.block_tile, *thread, td.rstep, td.traffic, td.smem_cost, td.block_per_SM, td.num_wave, td.grid_size]
+
+
+def orow(d):
+    thread = list(d["thread_tile"]) or [0, 0]
+    return [*d["block_tile"], *thread, d["rstep"], d["traffic"], d["smem_cost"], d["block_per_SM"], d["num_wave"], d["grid_size"]]
+
+
+# ---- 1. golden vectors from the reference ----------------------------------------------------
+
+def test_integer_helpers_match_reference_vectors(golden_policy):
+    u = golden_policy["utils"]
+    for n, expect in u["get_all_factors"].items():
+        assert utils.get_all_factors(int(n)) == expect
+        assert po.divisors(int(n)) == expect
+    for n, expect in u["factorize"].items():
+        assert utils.factorize(int(n)) == expect
+    for case in u["coalesced"]:
+        assert utils.coalesced_factor(case["sub"], case["full"]) == case["factor"]
+        assert utils.coalesced_tensor_shape(case["sub"], case["full"], case["txn"]) == case["shape"]
+        assert po.run_length(case["sub"], case["full"]) == case["factor"]
+        assert po.moved_elements(case["sub"], case["full"], case["txn"]) == case["shape"]
+    for case in u["get_block_dims"]:
+        assert utils.get_block_dims(case["block"], case["reg"]) == case["dims"]
+    for case in u["compute_memory_traffic"]:
+        cfg = MatmulConfig(case["M"], case["N"], case["K"], 32)
+        assert analyze.compute_memory_traffic(case["tile"], cfg, CUDA()) == case["bytes"]
+        assert po.tile_traffic(*case["tile"], case["M"], case["N"], case["K"]) == case["bytes"]
+
+
+def test_product_policy_reproduces_reference_hints(golden_policy):
+    assert len(golden_policy["shapes"]) == 20
+    for sh in golden_policy["shapes"]:
+        cfg = MatmulConfig(sh["M"], sh["N"], sh["K"], 32)
+        policy = Policy(cfg, CUDA())
+        assert policy._assign_reduce_step() == sh["base_rstep"]
+        assert policy.get_reduce_step_candidates(sh["K"]) == sh["reduce_step_candidates"]
+        ranked = policy.get_block_tiles_candidates([1, 1], sh["base_rstep"])
+        assert len(ranked) == sh["n_valid_block_tiles"]
+        assert [row(t) for t in ranked[:40]] == sh["ranked_block_tiles"]
+        for name, order in sh["block_sizes"].items():
+            tile = [int(v) for v in name.split("x")]
+            td = TileDict.from_block_tile(tile, sh["base_rstep"], cfg, CUDA())
+            assert policy.recommend_block_size(td) == order
+        hints = get_roller_hints(cfg, CUDA(), topk=20)
+        assert [row(h) for h in hints] == sh["hints"], (sh["M"], sh["N"], sh["K"])
+
+
+def test_policy_oracle_reproduces_reference_hints(golden_policy):
+    for sh in golden_policy["shapes"]:
+        M, N, K = sh["M"], sh["N"], sh["K"]
+        assert po.base_reduce_step(M, N, K) == sh["base_rstep"]
+        ranked = po.ranked_tiles(M, N, K)
+        assert len(ranked) == sh["n_valid_block_tiles"]
+        assert [orow(t) for t in ranked[:40]] == sh["ranked_block_tiles"]
+        assert [orow(h) for h in po.hints(M, N, K, 20)] == sh["hints"]
+        for name, order in sh["block_sizes"].items():
+            assert po.block_sizes(*[int(v) for v in name.split("x")]) == order
+
+
+# ---- 2. hand-derived known answers ---------------------------------------------------------------
+
+def test_closed_form_traffic():
+    # n >= 8 write-transaction elements: 4 * (K*(m+n) + m*n)
+    for (M, N, K), (m, n) in itertools.product([(2048, 2048, 2048), (4096, 8192, 4096)], [(128, 128), (64, 256), (32, 8)]):
+        cfg = MatmulConfig(M, N, K, 32)
+        assert analyze.compute_memory_traffic([m, n], cfg, CUDA()) == 4 * (K * (m + n) + m * n)
+    # narrower than a write transaction: each row of the tile costs a whole transaction (8 elems)
+    cfg = MatmulConfig(2048, 2048, 2048, 32)
+    assert analyze.compute_memory_traffic([64, 4], cfg, CUDA()) == 4 * (2048 * 68 + 8 * 64)
+
+
+def test_hand_derived_tile_analysis_a100():
+    cfg = MatmulConfig(2048, 2048, 2048, 32)
+    expect = {
+        (128, 128): (2162688, 32768, 4, 256, 1),
+        (64, 256): (2686976, 40960, 3, 256, 1),
+        (64, 64): (1064960, 16384, 4, 1024, 3),
+        (64, 128): (1605632, 24576, 4, 512, 2),
+        (128, 256): (3276800, 49152, 2, 128, 1),
+        (256, 256): (4456448, 65536, 2, 64, 1),
+    }
+    for tile, (traffic, smem, bps, grid, waves) in expect.items():
+        td = TileDict.from_block_tile(list(tile), 32, cfg, CUDA())
+        assert td.valid
+        assert (td.traffic, td.smem_cost, td.block_per_SM, td.grid_size, td.num_wave) == (traffic, smem, bps, grid, waves)
+    assert not TileDict.from_block_tile([512, 1], 32, cfg, CUDA()).valid  # 128 * 513 bytes > 64 KiB
+    big = TileDict.from_block_tile([4096, 8192], 1, MatmulConfig(8192, 8192, 64, 32), CUDA())
+    assert not big.valid and big.traffic == -1  # register estimate over the cap, analysis left unset
+
+
+def test_first_hint_a100_is_the_documented_one():
+    for shape in [(2048, 2048, 2048), (2048, 2048, 8192), (4096, 8192, 4096)]:
+        h = get_roller_hints(MatmulConfig(*shape, 32), CUDA(), topk=1)[0]
+        assert (h.block_tile, h.thread_tile, h.rstep, h.smem_cost, h.block_per_SM) == ([128, 128], [16, 8], 32, 32768, 4)
+        assert utils.get_block_dims(h.block_tile + [0], h.thread_tile + [0]) == [16, 8, 1]
+
+
+def test_reduce_step_expansion_and_thread_tiles_a100():
+    cfg = MatmulConfig(2048, 2048, 2048, 32)
+    policy = Policy(cfg, CUDA())
+    td = TileDict.from_block_tile([64, 64], 32, cfg, CUDA())
+    policy._expand_reduce_axis(td)
+    assert (td.rstep, td.smem_cost) == (64, 32768) and td.block_per_SM == 4  # occupancy not recomputed
+    td = TileDict.from_block_tile([128, 128], 32, cfg, CUDA())
+    policy._expand_reduce_axis(td)
+    assert td.rstep == 32
+    # [128,128]: 128 threads -> [16,8]; next block size 64 -> [16,16] needs 256 regs -> sequence ends
+    assert [t.thread_tile for t in policy.assign_thread_tile(td, 2)] == [[16, 8]]
+    assert policy.recommend_block_size(td)[:5] == [128, 64, 256, 32, 512]
+    assert policy.recommend_block_size(td)[-1] == 1024
+
+
+def test_large_prime_reduce_axis_uses_powers_of_two():
+    policy = Policy(MatmulConfig(64, 64, 127, 32), CUDA())
+    assert policy.get_reduce_step_candidates(127) == [1, 2, 4, 8, 16, 32, 64]
+    assert policy.get_reduce_step_candidates(61) == [1, 61]  # small prime: divisors kept
+
+
+def test_tiledict_hash_repr_and_clone():
+    cfg = MatmulConfig(2048, 2048, 2048, 32)
+    h = get_roller_hints(cfg, CUDA(), topk=2)
+    assert hash(h[0]) == hash(tuple(h[0].block_tile + h[0].thread_tile))
+    assert len({h[0]: 1, h[1]: 2}) == 2
+    text = repr(h[0])
+    assert "block_tile=[128, 128]" in text and "2.1 MiB" in text and "32.0 KiB" in text
+    twin = h[0].clone()
+    twin.block_tile[0] = 1
+    assert h[0].block_tile[0] == 128
+
+
+# ---- 3. product vs independent restatement on further shapes -----------------------------------
+
+def test_product_equals_restatement_on_random_shapes():
+    rng = random.Random(7)
+    dims = [48, 64, 96, 100, 127, 192, 250, 256, 384, 500, 512, 640, 1000, 1024, 1536, 3000]
+    for _ in range(25):
+        M, N, K = rng.choice(dims), rng.choice(dims), rng.choice(dims)
+        got = [row(h) for h in get_roller_hints(MatmulConfig(M, N, K, 32), CUDA(), topk=12)]
+        assert got == [orow(h) for h in po.hints(M, N, K, 12)], (M, N, K)
+
+
+def test_invariants_of_emitted_hints_a100():
+    for shape in [(2048, 4096, 2048), (3000, 5000, 1536), (1000, 640, 384)]:
+        cfg = MatmulConfig(*shape, 32)
+        arch = CUDA()
+        policy = Policy(cfg, arch)
+        base = policy._assign_reduce_step()
+        ranked = policy.get_block_tiles_candidates([1, 1], base)
+        prios = [(t.traffic + 1) * t.num_wave for t in ranked]
+        assert prios == sorted(prios)
+        for h in get_roller_hints(cfg, arch, topk=20):
+            m, n = h.block_tile
+            tm, tn = h.thread_tile
+            assert h.smem_cost == h.rstep * (m + n) * 4 <= arch.smem_cap
+            assert cfg.K % h.rstep == 0 and h.rstep % base == 0
+            assert (m * n) % (tm * tn) == 0 and tm >= tn and tm * tn < 256
+            assert h.grid_size == math.ceil(cfg.M / m) * math.ceil(cfg.N / n)
+
+
+# ---- MI355X model -------------------------------------------------------------------------------------
+
+def test_mi355x_model_numbers():
+    a = MI355X()
+    assert (a.compute_max_core, a.warp_size, a.sm_partition, a.xcd_count) == (256, 64, 4, 8)
+    assert a.reg_cap == 131072 and a.lds_bytes == 160 * 1024
+    assert a.smem_cap == a.max_smem_usage == 80 * 1024  # per pipeline stage under double buffering
+    assert a.get_avaliable_tensorintrin_shapes() == [(32, 32, 2), (16, 16, 4)]
+    # 256 CUs * 4 SIMDs * 64 FLOP/clk * 2.4 GHz
+    assert a.peak_matrix_tflops == pytest.approx(256 * 4 * 64 * 2.4e9 / 1e12, rel=1e-3)
+    with pytest.raises(NotImplementedError):
+        CUDA().get_avaliable_tensorintrin_shapes()
+    assert TileDevice().reg_estimate_divisor == 32 and TileDevice().thread_reg_limit == 256
+
+
+class _Props:
+    compute_units = 128
+    lds_bytes_per_block = 65536
+    clock_khz = 2000000
+    l2_bytes = 1 << 20
+
+
+def test_mi355x_from_device_overrides():
+    a = MI355X.from_device(_Props())
+    assert a.compute_max_core == 128 and a.smem_cap == 32768 and a.clock_mhz == 2000
+    assert a.peak_matrix_tflops == pytest.approx(128 * 256 * 2.0e9 / 1e12)
+
+
+SHAPES_MI = [(2048, 2048, 2048), (2048, 2048, 8192), (4096, 8192, 4096), (8192, 4096, 2048), (3000, 5000, 1536), (200, 300, 72)]
+
+
+@pytest.mark.parametrize("shape", SHAPES_MI)
+def test_mi355x_hints_are_launchable_kernel_configs(shape):
+    cfg = MatmulConfig(*shape, 32)
+    arch = MI355X()
+    hints = get_roller_hints(cfg, arch, topk=20)
+    assert 1 <= len(hints) <= 20
+    for h in hints:
+        m, n = h.block_tile
+        wm, wn = h.wave_tile
+        mi = h.mfma
+        assert mi in (32, 16) and m % wm == 0 and n % wn == 0 and wm % mi == 0 and wn % mi == 0
+        assert (wn // mi) in (1, 2) or (wn // mi) % 4 == 0
+        assert h.threads == 64 * (m // wm) * (n // wn) <= 1024
+        assert h.rstep % (4 * 64 // mi) == 0
+        # thread tile = wave tile seen per lane; launch geometry formula of the reference still holds
+        assert h.thread_tile == [wm // 8, wn // 8]
+        dims = utils.get_block_dims(h.block_tile + [0], h.thread_tile + [0])
+        assert dims[0] * dims[1] == h.threads
+        assert h.thread_tile[0] * h.thread_tile[1] <= 256          # accumulators per lane
+        assert h.smem_cost == (h.rstep * (m + n) + 4 * m) * 4         # one stage, LDS-A rows padded
+        assert 2 * h.smem_cost <= arch.lds_bytes                    # double-buffered tile fits a CU
+        g = hint_to_gemm_config(cfg, h, 2)
+        assert g.lds_bytes == 2 * h.smem_cost
+        assert h.grid_size == math.ceil(cfg.M / m) * math.ceil(cfg.N / n)
+
+
+def test_mi355x_ranking_prefers_tiles_that_fill_the_chip():
+    policy = Policy(MatmulConfig(2048, 2048, 2048, 32), MI355X())
+    by_tile = {tuple(t.block_tile): policy.estimate_seconds(t) for t in policy.get_block_tiles_candidates([1, 1], 32)}
+    # 256x256 leaves three quarters of the CUs idle on a 2048^2 output; 128x128 gives one tile per CU
+    assert by_tile[(128, 128)] < by_tile[(256, 128)] < by_tile[(256, 256)]
+    big = Policy(MatmulConfig(8192, 8192, 8192, 32), MI355X())
+    by_tile = {tuple(t.block_tile): big.estimate_seconds(t) for t in big.get_block_tiles_candidates([1, 1], 32)}
+    assert by_tile[(256, 256)] < by_tile[(32, 32)]
+    ranked = big.get_block_tiles_candidates([1, 1], 32)
+    est = [big.estimate_seconds(t) for t in ranked]
+    assert est == sorted(est)
+
+
+def test_mi355x_ragged_problem_gets_ladder_tiles():
+    policy = Policy(MatmulConfig(3000, 5000, 1536, 32), MI355X())
+    tiles = {tuple(t.block_tile) for t in policy.get_block_tiles_candidates([1, 1], 32)}
+    assert (128, 128) in tiles and (256, 256) in tiles     # neither divides 3000 or 5000
+    assert all(m % 16 == 0 and n % 16 == 0 for m, n in tiles)
+    assert all(s % 16 == 0 for s in policy.get_reduce_step_candidates(1536))
+    odd = Policy(MatmulConfig(37, 53, 29, 32), MI355X())
+    assert odd._assign_reduce_step() % 16 == 0
+    assert get_roller_hints(MatmulConfig(37, 53, 29, 32), MI355X(), topk=4)
+
+
+def test_split_block_over_waves():
+    a = MI355X()
+    assert analyze.split_block_over_waves([128, 128], 4, 32, a) == ([64, 64], 32)
+    assert analyze.split_block_over_waves([256, 256], 4, 32, a) == ([128, 128], 32)
+    assert analyze.split_block_over_waves([128, 128], 2, 32, a) == ([64, 128], 32)
+    assert analyze.split_block_over_waves([16, 64], 1, 16, a) == ([16, 64], 16)   # only the 16x16x4 shape fits
+    assert analyze.split_block_over_waves([48, 48], 1, 32, a) is None             # 3 column blocks: no vector read
+    assert analyze.split_block_over_waves([64, 64], 4, 8, a) == ([32, 32], 32)   # k step 8 rules out 16x16x4 only
