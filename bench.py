@@ -55,12 +55,53 @@ def blas_threads() -> int:
     return int(os.environ.get("OPENBLAS_NUM_THREADS") or os.environ.get("OMP_NUM_THREADS") or os.cpu_count() or 1)
 
 
+COPY_KERNEL = r"""
+extern "C" __global__ void copy_kernel(const float4* __restrict__ src, float4* __restrict__ dst, long n) {
+  for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+"""
+
+
+def copy_workload(args) -> int:
+    """Calibration workload for the HBM traffic counters: a plain copy of 256 MiB per launch
+    (256 MiB read, 256 MiB written), so that FETCH_SIZE / WRITE_SIZE of the GEMM kernel can be
+    scaled by what the same counters read for a known amount of traffic."""
+    import ctypes
+    from mlir_roller_amd import hip
+    from mlir_roller_amd.hip import DeviceArray, Event, Module, Stream
+
+    hip.init(0)
+    nbytes = 256 << 20
+    src = DeviceArray.from_host(np.ones(nbytes // 4, np.float32))
+    dst = DeviceArray.zeros((nbytes // 4,))
+    code, _ = hip.compile_source(COPY_KERNEL, "copy.hip")
+    func = Module(code).get_function("copy_kernel")
+    stream = Stream()
+    n16 = ctypes.c_long(nbytes // 16)
+    launch = lambda: func((4096,), (256,), (src, dst, n16), stream=stream)
+    for _ in range(args.warmup):
+        launch()
+    e0, e1 = Event(), Event()
+    e0.record(stream)
+    for _ in range(args.steps):
+        launch()
+    e1.record(stream)
+    e1.synchronize()
+    ms = hip.get_elapsed_time(e0, e1) / max(args.steps, 1)
+    ok = bool(np.all(dst.get() == 1.0))
+    print(json.dumps({"metric": "copy_kernel GB/s (read+write)", "value": round(2 * nbytes / ms / 1e6, 1), "unit": "GB/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 5),
+                      "config": {"workload": "copy: 256 MiB read + 256 MiB written per launch"},
+                      "bytes_read_per_launch": nbytes, "bytes_written_per_launch": nbytes, "ok": ok}), flush=True)
+    return 0 if ok else 1
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="sweep", help="sweep (M0..M13), one of M0..M13, or cfg4 (3000x5000x1536)")
+    ap.add_argument("--workload", default="sweep", help="sweep (M0..M13), one of M0..M13, cfg4 (3000x5000x1536), or copy (traffic-counter calibration)")
     ap.add_argument("--topk", type=int, default=20)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--retune", action="store_true", help="ignore remembered winners")
@@ -71,6 +112,9 @@ def main() -> int:
         print(f"bench.py: this build runs on ONE GPU (the GEMM path has no multi-GPU part); got --gpus {args.gpus}",
               file=sys.stderr)
         return 2
+
+    if args.workload == "copy":
+        return copy_workload(args)
 
     from mlir_roller_amd import hip
     from mlir_roller_amd.analyze import MatmulConfig, get_roller_hints
