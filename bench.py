@@ -119,7 +119,7 @@ def main() -> int:
     from mlir_roller_amd import hip
     from mlir_roller_amd.analyze import MatmulConfig, get_roller_hints
     from mlir_roller_amd.arch import MI355X
-    from mlir_roller_amd.benchmark import README_SHAPES
+    from mlir_roller_amd.benchmark import PIPELINE_DEPTH, README_SHAPES
     from mlir_roller_amd.hip import DeviceArray, Event, GemmConfig, GemmPlan, Stream
     from mlir_roller_amd.roller import gemm_errors, hint_to_gemm_config, make_inputs
 
@@ -144,7 +144,7 @@ def main() -> int:
     cache_dir = Path(os.environ.get("ROLLER_HIP_CACHE", str(hip.DEFAULT_CACHE_DIR)))
     cache_dir.mkdir(parents=True, exist_ok=True)
     template_id = hashlib.sha1(hip.template_source().encode()).hexdigest()[:12]
-    tuned_path = cache_dir / f"tuned_{template_id}_top{args.topk}.json"
+    tuned_path = cache_dir / f"tuned_{template_id}_top{args.topk}_d{PIPELINE_DEPTH}.json"
     tuned = {}
     if tuned_path.exists() and not args.retune:
         try:
@@ -188,7 +188,7 @@ def main() -> int:
             t0 = time.perf_counter()
             for rank, hint in enumerate(hints, 1):
                 try:
-                    g = hint_to_gemm_config(cfg, hint, 2)
+                    g = hint_to_gemm_config(cfg, hint, PIPELINE_DEPTH)
                     hip.config_check(g)
                     plan = GemmPlan(g)
                     compile_s += plan.compile_ms / 1e3
@@ -292,7 +292,7 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": workload, "launches_per_step": launches, "inputs": f"{dist}, seed {args.seed}",
-                   "topk": args.topk, "pipeline_depth": 2},
+                   "topk": args.topk, "pipeline_depth": PIPELINE_DEPTH},
         "pct_of_fp32_matrix_peak": round(100 * tflops / PEAK_TFLOPS, 2),
         "roofline": {
             "bound": "mfma", "achieved": round(tflops, 3), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",

@@ -62,7 +62,7 @@ typedef struct rl_gemm_config {
   int bk;          /* K step                <- hint.rstep                            */
   int wm, wn;      /* wave tile             <- 64 lanes x hint.thread_tile           */
   int mi;          /* 32: v_mfma_f32_32x32x2_f32, 16: v_mfma_f32_16x16x4_f32        */
-  int stages;      /* LDS buffers (1 or 2)  <- pipeline_depth                        */
+  int stages;      /* pipeline depth 1..3   <- pipeline_depth (2 LDS buffers from 2) */
   int pad_a, pad_b;/* LDS row padding in floats (multiples of 4)                     */
   int vec;         /* 4: 128-bit global accesses, 1: dword accesses (any K, N, ld)   */
   int edge;        /* 1: ragged tiles predicated, 0: bm|M, bn|N, bk|K required       */
@@ -131,7 +131,7 @@ int rl_sync(void);
 const char* rl_gemm_template_source(void);
 
 /* Checks cfg against the template's constraints without compiling.  *lds_bytes (may be NULL)
- * receives the dynamic LDS size = stages * (bm*(bk+pad_a) + bk*(bn+pad_b)) * 4, the padded
+ * receives the dynamic LDS size = min(stages,2) * (bm*(bk+pad_a) + bk*(bn+pad_b)) * 4, the padded
  * counterpart of hint.smem_cost * pipeline_depth (src/roller.py:385); *threads (may be NULL)
  * receives 64 * (bm/wm) * (bn/wn). */
 int rl_gemm_config_check(const rl_gemm_config* cfg, int* lds_bytes, int* threads);

@@ -196,14 +196,14 @@ def _similarity(a: float, b: float) -> float:
     return (2 * a * b) / (a * a + b * b)
 
 
-def split_block_over_waves(block_tile: List[int], waves: int, rstep: int, arch: TileDevice):
+def split_block_over_waves(block_tile: List[int], waves: int, rstep: int, arch: TileDevice, shapes=None):
     """Wave tile ``[wm, wn]`` and MFMA size for a block tile computed by ``waves`` wavefronts,
     or None.  A wave tile must be a grid of MFMA blocks whose column count the kernel reads
     with one vector load (1, 2 or a multiple of 4 blocks), and the reduce step must hold whole
     128-bit fragment reads (4 * wave / mi elements of k).  The larger instruction is preferred;
     among its wave tiles the most square wins, wider before taller."""
     m, n = block_tile
-    for shape in arch.mfma_shapes:
+    for shape in (arch.mfma_shapes if shapes is None else shapes):
         mi = shape[0]
         if rstep % (4 * arch.warp_size // mi):
             continue
@@ -232,6 +232,9 @@ class Policy:
     # tile sizes offered in addition to the exact divisors of a dimension
     SIMT_LADDER = (2, 4, 8, 16, 32)
     MFMA_LADDER = (16, 32, 64, 128, 256, 512)
+    # registers per lane the MFMA kernel needs besides its accumulators: two sets of operand
+    # fragments, the global->LDS staging registers and addresses (measured: 90-110)
+    REG_OVERHEAD = 96
 
     def __init__(self, config: MatmulConfig, arch: TileDevice) -> None:
         self.arch = arch
@@ -296,24 +299,23 @@ class Policy:
 
     def estimate_seconds(self, td: TileDict) -> float:
         """Roofline estimate of the whole GEMM with block tile ``td`` on a device with matrix
-        cores.  The busiest CU works through ceil(grid / CUs) tiles one after another; a tile
-        costs the larger of its MFMA time at the CU's share of the matrix peak and its traffic
-        at the CU's share of the memory bandwidth, plus a fixed cost for filling the pipeline
-        and draining the accumulators that does not shrink with the tile."""
+        cores.  The busiest CU works through ceil(grid / CUs) tiles one after another.  A tile
+        costs the larger of its MFMA time at the CU's share of the matrix peak and its traffic at
+        the CU's share of the memory bandwidth.  MFMA time is divided by an issue efficiency that
+        falls with the operand traffic per FLOP, (1/m + 1/n): fitted to measurements on MI355X
+        (about 0.95 for 256x256 tiles, 0.81 for 32x64).  A fixed cost per tile covers filling the
+        pipeline and draining the accumulators."""
         a, cfg = self.arch, self.matmul_config
         m, n = td.block_tile
         cu_flops = a.peak_matrix_tflops * 1e12 / a.compute_max_core
         cu_bw = a.bandwidth[0] * 1e9 / a.compute_max_core
-        # padded work: the kernel runs whole MFMA tiles also where the problem is ragged
-        k_steps = -(-cfg.K // td.rstep)
-        t_mfma = 2.0 * m * n * k_steps * td.rstep / cu_flops
+        k_steps = -(-cfg.K // td.rstep)  # the kernel runs whole K steps also where K is ragged
+        efficiency = max(0.972 - 3.456 * (1.0 / m + 1.0 / n), 0.05)
+        t_mfma = 2.0 * m * n * k_steps * td.rstep / (cu_flops * efficiency)
         t_mem = td.traffic / cu_bw
-        # one reduce step of latency exposed at start-up, and the C tile written at the end
-        t_fixed = 2.0e-6 + m * n * cfg.el_bytes / cu_bw
+        t_fixed = 1.0e-6 + m * n * cfg.el_bytes / cu_bw
         tiles_per_cu = -(-td.grid_size // a.compute_max_core)
-        # small wave tiles re-read their LDS fragments more often per MFMA; charge it mildly
-        reuse_penalty = 1.0 + 8.0 / (m + n)
-        return tiles_per_cu * (max(t_mfma * reuse_penalty, t_mem) + t_fixed)
+        return tiles_per_cu * (max(t_mfma, t_mem) + t_fixed)
 
     def get_block_tiles_candidates(self, init_tile: List[int], rstep: int) -> List[TileDict]:
         """All valid block tiles, best first (stable with respect to enumeration order:
@@ -352,7 +354,7 @@ class Policy:
     def score_block_size(self, n: int):
         """(distance of the warp count from one warp per scheduler, fraction of idle lanes in
         the last warp); smaller is better."""
-        warp, part = self.arch.warp_size, self.arch.sm_partition
+        warp, part = self.arch.warp_size, self.arch.sm_partition * self.arch.waves_per_partition
         warps = -(-n // warp)
         return (max(warps / part, part / warps), (warps * warp - n) / n)
 
@@ -362,20 +364,30 @@ class Policy:
         return sorted(sizes, key=self.score_block_size)
 
     def assign_thread_tile(self, td: TileDict, topk: int = 1) -> Iterator[TileDict]:
-        """Yields up to ``topk`` completed copies of ``td``, one per block size in recommended
-        order.  The first block size that cannot be tiled ends the sequence."""
+        """Yields completed copies of ``td`` for up to ``topk`` block sizes in recommended order.
+        Without matrix cores the first block size that cannot be tiled ends the sequence (the
+        reference's behaviour).  With matrix cores such a block size is skipped -- most thread
+        counts are not a whole number of waves or do not split into MFMA blocks -- and a block
+        size that works yields one copy per matrix-instruction shape that fits."""
         for block_size in self.recommend_block_size(td):
-            done = self._assign_thread_tile(td, block_size)
-            if done is None:
-                return
-            yield done
+            if self.arch.has_matrix_cores:
+                done = self._assign_wave_tiles(td, block_size)
+                if not done:
+                    continue
+                yield from done
+            else:
+                one = self._assign_thread_tile(td, block_size)
+                if one is None:
+                    return
+                yield one
             topk -= 1
             if topk == 0:
                 return
 
     def _assign_thread_tile(self, td: TileDict, block_size: int) -> Optional[TileDict]:
         if self.arch.has_matrix_cores:
-            return self._assign_wave_tile(td, block_size)
+            done = self._assign_wave_tiles(td, block_size)
+            return done[0] if done else None
         area = math.prod(td.block_tile) // block_size
         pairs = [[area // i, i] for i in range(1, math.isqrt(area) + 1) if area % i == 0]
         k, lds_bw = self.matmul_config.K, self.arch.bandwidth[1]
@@ -387,27 +399,39 @@ class Policy:
         td.thread_tile = best
         return td.clone()
 
-    def _assign_wave_tile(self, td: TileDict, block_size: int) -> Optional[TileDict]:
+    def _assign_wave_tiles(self, td: TileDict, block_size: int) -> List[TileDict]:
         """The thread-tile step on a device with matrix cores: the block tile is split over
-        ``block_size / wave`` wavefronts (see ``split_block_over_waves``)."""
-        warp = self.arch.warp_size
+        ``block_size / wave`` wavefronts, once per matrix-instruction shape that admits a split
+        (``split_block_over_waves``).  A split is dropped when its accumulators, plus room for
+        operand fragments and staging, exceed the registers a lane can address at the number of
+        waves this block puts on each SIMD."""
+        arch = self.arch
+        warp = arch.warp_size
         if block_size % warp:
-            return None
-        split = split_block_over_waves(td.block_tile, block_size // warp, td.rstep, self.arch)
-        if split is None:
-            return None
-        wave_tile, mi = split
+            return []
+        waves = block_size // warp
         lanes_side = math.isqrt(warp)  # 64 lanes seen as 8 x 8
-        if wave_tile[0] % lanes_side or wave_tile[1] % lanes_side:
-            return None
-        thread_tile = [wave_tile[0] // lanes_side, wave_tile[1] // lanes_side]
-        if int(math.prod(thread_tile) * self.matmul_config.el_bytes / 4) >= self.arch.thread_reg_limit:
-            return None
-        td.thread_tile = thread_tile
-        td.wave_tile = wave_tile
-        td.mfma = mi
-        td.threads = block_size
-        return td.clone()
+        budget = arch.regs_per_lane // max(1, -(-waves // arch.sm_partition)) if arch.regs_per_lane else 0
+        out: List[TileDict] = []
+        for shape in arch.mfma_shapes:
+            split = split_block_over_waves(td.block_tile, waves, td.rstep, arch, shapes=[shape])
+            if split is None:
+                continue
+            wave_tile, mi = split
+            if wave_tile[0] % lanes_side or wave_tile[1] % lanes_side:
+                continue
+            thread_tile = [wave_tile[0] // lanes_side, wave_tile[1] // lanes_side]
+            acc_regs = int(math.prod(thread_tile) * self.matmul_config.el_bytes / 4)
+            if acc_regs >= arch.thread_reg_limit:
+                continue
+            if budget and acc_regs + self.REG_OVERHEAD > budget:
+                continue
+            td.thread_tile = thread_tile
+            td.wave_tile = wave_tile
+            td.mfma = mi
+            td.threads = block_size
+            out.append(td.clone())
+        return out
 
     # ---- top level ------------------------------------------------------------------------------
 

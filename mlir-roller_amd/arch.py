@@ -38,6 +38,10 @@ class TileDevice:
     thread_reg_limit: int = 256
     # elements of padding the kernel adds to every row of the [m, rstep] workgroup-memory tile
     lds_row_pad: int = 0
+    # warps per scheduler that the block-size recommendation aims for
+    waves_per_partition: int = 1
+    # 32-bit registers one lane can address when a scheduler hosts a single warp (0 = not modelled)
+    regs_per_lane: int = 0
     # matrix-instruction shapes (m, n, k); empty = no matrix cores modelled, SIMT outer product
     mfma_shapes: List[Tuple[int, int, int]] = field(default_factory=list)
     # dies with a private L2 that the dispatcher deals workgroups to round-robin
@@ -106,6 +110,10 @@ class MI355X(TileDevice):
     # rows of the LDS A tile are padded by one 16-byte unit so that 128-bit reads of
     # consecutive rows fall into distinct bank groups
     lds_row_pad: int = 4
+    # two waves per SIMD let one wave's LDS traffic and barriers hide behind the other's MFMAs
+    waves_per_partition: int = 2
+    # 256 architectural + 256 accumulation registers per lane, shared by the waves of a SIMD
+    regs_per_lane: int = 512
     mfma_shapes: List[Tuple[int, int, int]] = field(default_factory=lambda: [(32, 32, 2), (16, 16, 4)])
     xcd_count: int = 8
     peak_matrix_tflops: float = 157.3

@@ -25,6 +25,8 @@ from .analyze import MatmulConfig, get_roller_hints
 from .arch import MI355X, TileDevice
 from .roller import Compiler, run_baseline, run_eval
 
+PIPELINE_DEPTH = 3
+
 # The fourteen shapes of the reference's result table, M0..M13 as (M, N, K) (README.md:13-17).
 README_SHAPES: List[Tuple[int, int, int]] = [
     (2048, 2048, 2048), (2048, 2048, 8192), (2048, 4096, 2048), (2048, 4096, 4096),
@@ -59,7 +61,8 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
                 baseline_time, baseline_gflops = float("inf"), 0
 
         # 2. roller hints
-        pipeline_depth = 2
+        # the reference runs depth 2 (benchmark.py:29); here 3 = two LDS buffers + a register stage
+        pipeline_depth = PIPELINE_DEPTH
         print(f"Generating and testing {topk} roller hints...")
         t0 = time.perf_counter()
         try:

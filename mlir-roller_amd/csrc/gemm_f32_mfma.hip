@@ -18,7 +18,11 @@
 //   BK          K step per main-loop iteration; multiple of 4*(64/MI)
 //   WM, WN      wave tile; (BM/WM)*(BN/WN) waves of 64 lanes form the workgroup
 //   MI          32 -> v_mfma_f32_32x32x2_f32, 16 -> v_mfma_f32_16x16x4_f32
-//   STAGES      LDS buffers: 2 = double buffer (one barrier per K step), 1 = single buffer
+//   STAGES      pipeline depth: 1 = one LDS buffer, nothing overlapped; 2 = two LDS buffers, the
+//               global loads of step k+1 in flight during the MFMAs of step k; 3 = two LDS buffers
+//               plus a register stage: global loads run two steps ahead, and the LDS fragments of
+//               the next MFMA group are read while the current group executes, also across the
+//               barrier that ends a K step
 //   PAD_A,PAD_B extra floats per LDS row of the A tile ([BM][BK+PAD_A]) and B tile ([BK][BN+PAD_B])
 //   VEC         4 = 128-bit global accesses (needs K%4==0, N%4==0, lda/ldb/ldc%4==0 and 16-byte
 //               aligned base pointers), 1 = dword accesses with per-element predicates
@@ -94,6 +98,9 @@
 #ifndef ACCUM
 #define ACCUM 0
 #endif
+#ifndef SCHED
+#define SCHED 1
+#endif
 
 #define NWM (BM / WM)
 #define NWN (BN / WN)
@@ -110,6 +117,8 @@
 #define A_STAGE (BM * LDA_S)
 #define B_STAGE (BK * LDB_S)
 #define STAGE_FLOATS (A_STAGE + B_STAGE)
+#define LDS_BUFS (STAGES >= 2 ? 2 : 1)
+#define SUPERS (BK / KSUPER) /* MFMA groups per K step, each fed by one round of fragment reads */
 #define A_UNITS (BM * BK / 4)
 #define B_UNITS (BK * BN / 4)
 #define A_PER_T ((A_UNITS + NT - 1) / NT)
@@ -123,9 +132,9 @@ static_assert(TN == 1 || TN == 2 || TN % 4 == 0, "column blocks per wave: 1, 2 o
 static_assert(BK % KSUPER == 0, "BK must be a multiple of 4*(64/MI)");
 static_assert(PAD_A % 4 == 0 && PAD_B % 4 == 0, "LDS rows stay 16-byte aligned");
 static_assert(NT <= 1024, "at most 16 waves per workgroup");
-static_assert(STAGES == 1 || STAGES == 2, "one or two LDS buffers");
+static_assert(STAGES >= 1 && STAGES <= 3, "pipeline depth 1, 2 or 3");
 static_assert(VEC == 4 || VEC == 1, "global access width");
-static_assert(STAGES * STAGE_FLOATS * 4 <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
+static_assert(LDS_BUFS * STAGE_FLOATS * 4 <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
 
 typedef float v2f __attribute__((ext_vector_type(2)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -156,6 +165,34 @@ typedef float bvec_t;
 #endif
 
 #define DEV static __device__ __forceinline__
+
+template <int V>
+struct int_c {
+  static constexpr int value = V;
+};
+
+// Instruction-scheduler directive: in the enclosing scheduling region, order the next NM MFMAs
+// and the next NO instructions of class MASK (0x100 LDS read, 0x200 LDS write, 0x020 global
+// read) so that the others are spread over the MFMAs as evenly as possible, earliest first:
+// each memory instruction is issued in the shadow of an MFMA instead of in a burst that leaves
+// the matrix pipe idle.
+template <int NM, int NO, int MASK>
+DEV void interleave_with_mfma() {
+  if constexpr (NM > 0) {
+    constexpr int q = NO / NM, rem = NO % NM;
+#pragma unroll
+    for (int i = 0; i < NM; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      if (i < rem) {
+        __builtin_amdgcn_sched_group_barrier(MASK, q + 1, 0);
+      } else if (q > 0) {
+        __builtin_amdgcn_sched_group_barrier(MASK, q > 0 ? q : 1, 0);
+      }
+    }
+  } else if constexpr (NO > 0) {
+    __builtin_amdgcn_sched_group_barrier(MASK, NO > 0 ? NO : 1, 0);
+  }
+}
 
 // Raw buffer resource over [base, base+bytes): loads beyond it return 0, stores beyond it are
 // dropped.  Word 3 = 0x00020000 is the 32-bit raw data format on gfx9-family targets.
@@ -260,10 +297,16 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 
   v4f ra[A_PER_T], rb[B_PER_T];
 
+  const int KT = (K + BK - 1) / BK;
+
+  // Issues the global loads of K step kt into the staging registers.  A step at or beyond KT
+  // (the pipelined loop asks for up to two steps ahead) gets an empty resource: every load
+  // returns 0 and touches no memory.
   auto fetch = [&](int kt) {
     const int k0 = kt * BK;
-    const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, a_rem - (long)k0 * 4);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + (long)k0 * ldb, b_rem - (long)k0 * ldb * 4);
+    const bool live = kt < KT;
+    const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, live ? a_rem - (long)k0 * 4 : 0);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + (long)k0 * ldb, live ? b_rem - (long)k0 * ldb * 4 : 0);
 #pragma unroll
     for (int i = 0; i < A_PER_T; ++i) {
       const int k = k0 + a_kcol[i];
@@ -301,37 +344,127 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   const int a_frag = (wm0 + lr) * LDA_S + 4 * lg;   // + bi*MI*LDA_S + kk
   const int b_frag = (4 * lg) * LDB_S + wn0 + VN * lr;  // + (kk+t)*LDB_S + v*MI*VN
 
-  auto multiply = [&](int stage) {
+  // One round of LDS fragment reads: TM 128-bit reads of A (four consecutive k each) and, for each
+  // of the four k slots, NVB vector reads of B.  Feeds 4*TM*TN MFMAs.
+  struct frag_t {
+    v4f a[TM];
+    bvec_t b[4][NVB];
+  };
+  auto read_frags = [&](frag_t& f, int stage, int kk) {
     const float* As = lds + stage * STAGE_FLOATS;
     const float* Bs = As + A_STAGE;
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += KSUPER) {
-      v4f af[TM];
+    for (int bi = 0; bi < TM; ++bi) f.a[bi] = *(const v4f*)&As[a_frag + bi * MI * LDA_S + kk];
 #pragma unroll
-      for (int bi = 0; bi < TM; ++bi) af[bi] = *(const v4f*)&As[a_frag + bi * MI * LDA_S + kk];
+    for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        bvec_t bf[NVB];
+      for (int v = 0; v < NVB; ++v) f.b[t][v] = *(const bvec_t*)&Bs[b_frag + (kk + t) * LDB_S + v * MI * VN];
+  };
+  auto mfma_frags = [&](const frag_t& f, int t0 = 0, int t1 = 4) {
 #pragma unroll
-        for (int v = 0; v < NVB; ++v)
-          bf[v] = *(const bvec_t*)&Bs[b_frag + (kk + t) * LDB_S + v * MI * VN];
+    for (int t = t0; t < t1; ++t)
 #pragma unroll
-        for (int bi = 0; bi < TM; ++bi)
+      for (int bi = 0; bi < TM; ++bi)
 #pragma unroll
-          for (int bj = 0; bj < TN; ++bj) {
+        for (int bj = 0; bj < TN; ++bj) {
 #if VN == 1
-            const float bval = bf[bj];
+          const float bval = f.b[t][bj];
 #else
-            const float bval = bf[bj / VN][bj % VN];
+          const float bval = f.b[t][bj / VN][bj % VN];
 #endif
-            acc[bi][bj] = MFMA(af[bi][t], bval, acc[bi][bj]);
-          }
-      }
-    }
+          acc[bi][bj] = MFMA(f.a[bi][t], bval, acc[bi][bj]);
+        }
   };
 
   // ---- main loop ----
-  const int KT = (K + BK - 1) / BK;
+#if STAGES == 3
+  if (KT > 0) {
+    // Software pipeline.  At the top of step kt: tile kt is in LDS buffer kt&1, its first fragment
+    // round is already in registers, and the staging registers hold tile kt+1 (loaded during step
+    // kt-1).  Within the step each fragment round is read while the previous one is in the MFMA
+    // pipe; before the last round is multiplied, tile kt+1 goes to the other LDS buffer, the
+    // loads of tile kt+2 are issued, the workgroup meets at the barrier, and the first fragment
+    // round of tile kt+1 is read -- so that the last MFMA group covers that read's latency.
+    frag_t fr[2];
+    fetch(0);
+    stash(0);
+    fetch(1);
+    __syncthreads();
+    read_frags(fr[0], 0, 0);
+
+    // P = which of the two fragment sets holds round 0 of this step (compile-time, so that the
+    // sets stay in fixed registers); the set alternates every round.
+    // MFMAs and fragment reads per round; LDS writes and global loads per K step
+    constexpr int G = 4 * TM * TN, R = TM + 4 * NVB, W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
+
+    auto step = [&](auto parity, int kt) {
+      constexpr int P = decltype(parity)::value;
+      const int cur = kt & 1;
+#pragma unroll
+      for (int r = 0; r + 1 < SUPERS; ++r) {
+        read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
+        mfma_frags(fr[(P + r) & 1]);
+      }
+      // the last round is split around the barrier: its first half covers the LDS writes of
+      // tile kt+1 and the global loads of tile kt+2, its second half the first reads of tile kt+1
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
+      stash(cur ^ 1);
+      fetch(kt + 2);
+#if SCHED
+#pragma unroll
+      for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
+      interleave_with_mfma<G / 4, W, 0x200>();
+      interleave_with_mfma<G / 2 - G / 4, L, 0x020>();
+#endif
+      __syncthreads();
+      read_frags(fr[(P + SUPERS) & 1], cur ^ 1, 0);
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 2, 4);
+#if SCHED
+      interleave_with_mfma<G / 2, R, 0x100>();
+#endif
+    };
+    auto last_step = [&](auto parity, int kt) {
+      constexpr int P = decltype(parity)::value;
+      const int cur = kt & 1;
+#pragma unroll
+      for (int r = 0; r + 1 < SUPERS; ++r) {
+        read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
+        mfma_frags(fr[(P + r) & 1]);
+      }
+      mfma_frags(fr[(P + SUPERS - 1) & 1]);
+#if SCHED
+#pragma unroll
+      for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
+#endif
+    };
+
+    int kt = 0;
+    if constexpr (SUPERS % 2 == 0) {
+      for (; kt < KT - 1; ++kt) step(int_c<0>{}, kt);
+      last_step(int_c<0>{}, kt);
+    } else {
+      // an odd number of rounds per step flips the parity every step: unroll by two
+      for (; kt + 1 < KT - 1; kt += 2) {
+        step(int_c<0>{}, kt);
+        step(int_c<1>{}, kt + 1);
+      }
+      if (kt < KT - 1) {
+        step(int_c<0>{}, kt);
+        last_step(int_c<1>{}, kt + 1);
+      } else {
+        last_step(int_c<0>{}, kt);
+      }
+    }
+  }
+#else
+  auto multiply = [&](int stage) {
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += KSUPER) {
+      frag_t f;
+      read_frags(f, stage, kk);
+      mfma_frags(f);
+    }
+  };
   if (KT > 0) {
     fetch(0);
     stash(0);
@@ -353,6 +486,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     __syncthreads();
 #endif
   }
+#endif
 
   // ---- epilogue: every accumulator leaves once ----
   float* Cg = C + (long)m0 * ldc + n0;

@@ -111,14 +111,14 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
   if (c.bk % ksuper) return fail(RL_ERR_INVALID_ARG, "bk must be a multiple of %d for mi=%d, got %d", ksuper, c.mi, c.bk);
   if (c.pad_a < 0 || c.pad_b < 0 || c.pad_a % 4 || c.pad_b % 4)
     return fail(RL_ERR_INVALID_ARG, "pad_a/pad_b must be non-negative multiples of 4");
-  if (c.stages != 1 && c.stages != 2) return fail(RL_ERR_INVALID_ARG, "stages must be 1 or 2, got %d", c.stages);
+  if (c.stages < 1 || c.stages > 3) return fail(RL_ERR_INVALID_ARG, "stages must be 1, 2 or 3, got %d", c.stages);
   if (c.vec != 4 && c.vec != 1) return fail(RL_ERR_INVALID_ARG, "vec must be 4 or 1, got %d", c.vec);
   if ((c.edge | 1) != 1 || (c.accum | 1) != 1) return fail(RL_ERR_INVALID_ARG, "edge and accum are 0 or 1");
   if (c.swz < 0 || c.swz > 3) return fail(RL_ERR_INVALID_ARG, "swz is a 2-bit mask");
   if ((c.swz & 2) && c.group <= 0) return fail(RL_ERR_INVALID_ARG, "group must be positive");
   const int nt = 64 * (c.bm / c.wm) * (c.bn / c.wn);
   if (nt > 1024) return fail(RL_ERR_INVALID_ARG, "%d threads per workgroup exceed 1024", nt);
-  const long lds = (long)c.stages * ((long)c.bm * (c.bk + c.pad_a) + (long)c.bk * (c.bn + c.pad_b)) * 4;
+  const long lds = (long)(c.stages >= 2 ? 2 : 1) * ((long)c.bm * (c.bk + c.pad_a) + (long)c.bk * (c.bn + c.pad_b)) * 4;
   if (lds > 160 * 1024) return fail(RL_ERR_INVALID_ARG, "%ld bytes of LDS exceed the 160 KB of a CU", lds);
   if (lds_bytes) *lds_bytes = (int)lds;
   if (threads) *threads = nt;
@@ -144,7 +144,7 @@ int compile(const char* source, const char* name, const std::vector<std::string>
             std::vector<char>* code, std::string* log) {
   // Fixed part of the command line: the one target this library serves, and no packed-fp32
   // instruction selection.
-  std::vector<std::string> all = {"--offload-arch=gfx950", "-O3", "-Xclang", "-target-feature",
+  std::vector<std::string> all = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
                                   "-Xclang", "-packed-fp32-ops"};
   all.insert(all.end(), user_opts.begin(), user_opts.end());
   std::vector<const char*> argv;

@@ -92,7 +92,7 @@ class GemmConfig:
 
     @property
     def lds_bytes(self) -> int:
-        return self.stages * (self.bm * (self.bk + self.pad_a) + self.bk * (self.bn + self.pad_b)) * 4
+        return min(self.stages, 2) * (self.bm * (self.bk + self.pad_a) + self.bk * (self.bn + self.pad_b)) * 4
 
     def tag(self) -> str:
         return (f"b{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_mi{self.mi}_s{self.stages}"

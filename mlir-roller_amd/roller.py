@@ -39,8 +39,8 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
     """Template parameters for one hint.
 
     block_tile -> BM, BN; rstep -> BK; wave_tile -> WM, WN (derived from the thread count when
-    the hint comes from a device model without matrix cores); pipeline_depth -> LDS buffers
-    (the template has 1 or 2).  Ragged problems switch on predication, and problems whose K, N
+    the hint comes from a device model without matrix cores); pipeline_depth -> pipeline stages
+    (the template has 1 to 3; from 2 on it keeps two LDS buffers).  Ragged problems switch on predication, and problems whose K, N
     are not multiples of 4 fall back to dword global accesses.
     """
     bm, bn = hint.block_tile
@@ -63,7 +63,7 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
     pad_a = 4 if (bk // 4) % 2 == 0 else 0
     return GemmConfig(
         bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi,
-        stages=max(1, min(2, int(pipeline_depth))), pad_a=pad_a, pad_b=0,
+        stages=max(1, min(3, int(pipeline_depth))), pad_a=pad_a, pad_b=0,
         vec=4 if (K % 4 == 0 and N % 4 == 0) else 1,
         edge=0 if (M % bm == 0 and N % bn == 0 and K % bk == 0) else 1,
         swz=3, group=8, accum=1 if accumulate else 0,
@@ -303,7 +303,7 @@ def run_baseline(config: MatmulConfig, repeat_times: int = 3, seed: int = 0):
 if __name__ == "__main__":
     S = 4096
     config = MatmulConfig(M=S, N=S, K=S, el_bits=32)
-    pipeline_depth = 2
+    pipeline_depth = 3
     hints = get_roller_hints(config, MI355X(), topk=20)
     run_baseline(config)
     timings = {}

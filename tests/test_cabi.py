@@ -52,7 +52,7 @@ def test_config_check_accepts_and_sizes(hip_lib):
     (dict(wm=48), "does not divide block tile"),
     (dict(wm=64, wn=64, bm=64, bn=64, mi=32, bk=12), "bk must be a multiple"),
     (dict(bm=96, bn=96, wm=96, wn=96), "wn/mi must be 1, 2 or a multiple of 4"),
-    (dict(stages=3), "stages must be"),
+    (dict(stages=4), "stages must be"),
     (dict(vec=2), "vec must be"),
     (dict(pad_a=2), "pad_a/pad_b"),
     (dict(bm=512, bn=512, wm=128, wn=128, bk=64), "exceed"),

@@ -16,12 +16,14 @@ def test_hint_to_gemm_config_aligned_problem():
     cfg = MatmulConfig(4096, 8192, 4096, 32)
     hint = next(h for h in get_roller_hints(cfg, MI355X(), 20) if h.block_tile == [256, 256])
     g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=2)
-    assert (g.bm, g.bn, g.bk, g.wm, g.wn, g.mi) == (256, 256, hint.rstep, 128, 128, 32)
+    assert (g.bm, g.bn, g.bk, g.wm, g.wn, g.mi) == (256, 256, hint.rstep, *hint.wave_tile, hint.mfma)
     assert (g.stages, g.vec, g.edge, g.accum) == (2, 4, 0, 0)
     assert ((g.bk + g.pad_a) // 4) % 2 == 1          # odd number of 16-byte units per LDS-A row
     assert g.threads == hint.threads and g.lds_bytes <= 160 * 1024
     assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=1).stages == 1
-    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=5).stages == 2
+    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).stages == 3
+    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=5).stages == 3
+    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).lds_bytes == g.lds_bytes   # still two LDS buffers
     assert roller.hint_to_gemm_config(cfg, hint, accumulate=True).accum == 1
 
 
