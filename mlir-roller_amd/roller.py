@@ -32,6 +32,7 @@ KERNEL_NAME = "gemm_kernel"  # the symbol the reference looks up (roller.py:499)
 # numerical gates of the GEMM path
 NORMWISE_TOL = 1e-5          # ||C - C32||_F / ||C32||_F against a float32 host GEMM
 ELEMENTWISE_FACTOR = 1e-4    # max|C - C64| <= factor * sqrt(K) * max|A| * max|B| against float64
+WARMUP_MS = 40.0             # load queued ahead of the timed launches of run_eval
 
 
 def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: int = 2,
@@ -240,7 +241,8 @@ def _host_case(config: MatmulConfig, seed: int, distribution: str):
 def run_eval(cuda_func: KernelHandle, pipeline_depth, hint: TileDict, repeat_times: int = 20,
              seed: int = 0, distribution: str = "uniform", check: bool = True):
     """Protocol of the reference's ``run_eval`` (roller.py:525-586): one checked launch, one
-    more single launch, ten warm-ups, then ``repeat_times`` launches between two events.
+    more single launch, warm-ups (ten, or as many as fill ``WARMUP_MS``), then ``repeat_times``
+    launches between two events.
     Returns ``(ms_per_launch, gflops)``; details land in ``cuda_func.last_eval``.
 
     Unlike the reference, which only prints on a mismatch, a result outside the tolerances
@@ -267,7 +269,11 @@ def run_eval(cuda_func: KernelHandle, pipeline_depth, hint: TileDict, repeat_tim
             raise AssertionError(f"GEMM result outside tolerance for {hint}: {info}")
 
     cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
-    for _ in range(10):
+    # The reference warms up with 10 launches.  On MI355X the engine clock drops as soon as the
+    # GPU idles (here: during the check above) and needs about 25 ms of load to come back, so
+    # the warm-up is extended to cover WARMUP_MS; it runs straight into the timed launches.
+    est_ms = 2.0 * M * N * K / 120e9
+    for _ in range(max(10, int(WARMUP_MS / est_ms) + 1)):
         cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
     with time_cuda() as (start_gpu, end_gpu):
         for _ in range(repeat_times):

@@ -274,3 +274,33 @@ def test_split_block_over_waves():
     assert analyze.split_block_over_waves([16, 64], 1, 16, a) == ([16, 64], 16)   # only the 16x16x4 shape fits
     assert analyze.split_block_over_waves([48, 48], 1, 32, a) is None             # 3 column blocks: no vector read
     assert analyze.split_block_over_waves([64, 64], 4, 8, a) == ([32, 32], 32)   # k step 8 rules out 16x16x4 only
+
+
+def test_mi355x_block_sizes_aim_for_two_waves_per_simd():
+    cfg = MatmulConfig(4096, 8192, 4096, 32)
+    policy = Policy(cfg, MI355X())
+    td = TileDict.from_block_tile([256, 256], 32, cfg, MI355X())
+    assert policy.recommend_block_size(td)[:3] == [512, 256, 1024]      # 8 waves, then 4 and 16 (tie: smaller first)
+    assert Policy(cfg, CUDA()).recommend_block_size(TileDict.from_block_tile([128, 128], 32, cfg, CUDA()))[0] == 128
+    hints = get_roller_hints(cfg, MI355X(), topk=4)
+    # one block tile, two block sizes, both matrix-instruction shapes
+    assert [(h.block_tile, h.wave_tile, h.threads, h.mfma) for h in hints] == [
+        ([256, 256], [64, 128], 512, 32), ([256, 256], [64, 128], 512, 16),
+        ([256, 256], [128, 128], 256, 32), ([256, 256], [128, 128], 256, 16)]
+
+
+def test_mi355x_register_budget_drops_splits_that_would_spill():
+    arch = MI355X()
+    for shape in SHAPES_MI + [(8192, 8192, 8192)]:
+        for h in get_roller_hints(MatmulConfig(*shape, 32), arch, topk=40):
+            waves_per_simd = -(-(h.threads // 64) // arch.sm_partition)
+            acc = h.thread_tile[0] * h.thread_tile[1]
+            assert acc + Policy.REG_OVERHEAD <= arch.regs_per_lane // waves_per_simd, h
+    cfg = MatmulConfig(8192, 8192, 8192, 32)
+    policy = Policy(cfg, arch)
+    assert not TileDict.from_block_tile([512, 256], 16, cfg, arch).valid   # 131072 accumulators fill the CU's registers
+    td = TileDict.from_block_tile([256, 256], 32, cfg, arch)
+    assert [h.threads for h in policy._assign_wave_tiles(td, 256)] == [256, 256]   # 256 + 96 <= 512
+    assert [h.threads for h in policy._assign_wave_tiles(td, 512)] == [512, 512]   # 128 + 96 <= 256
+    assert policy._assign_wave_tiles(td, 1024) == []                               # 64 + 96 > 128
+    assert policy._assign_wave_tiles(td, 96) == []                                 # not a whole number of waves
