@@ -38,6 +38,11 @@ sys.path.insert(0, str(ROOT))
 import numpy as np  # noqa: E402
 
 PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak: 256 CUs * 256 FLOP/clk * 2.4 GHz
+# HBM-side bytes per launch (L2 misses, Infinity-Cache hits included) of the winning kernels,
+# measured offline with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE in separate runs and scaled by
+# what the same counters read for a 256 MiB copy kernel (FETCH_SIZE x2.0, WRITE_SIZE x1.0).
+# "sweep" is the mean over one pass of the 14 shapes; algorithmic bytes are 226.5 MB resp. 335.5 MB.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"sweep": 544.4e6, "M10": 939.6e6}
 RAMP_MS = 40.0       # continuous load queued ahead of every timed region (engine-clock ramp)
 
 
@@ -307,7 +312,7 @@ def main() -> int:
         "pct_of_fp32_matrix_peak": round(100 * tflops / PEAK_TFLOPS, 2),
         "roofline": {
             "bound": "mfma", "achieved": round(tflops, 3), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": round(tflops / PEAK_TFLOPS, 4), "traffic": None,
+            "frac": round(tflops / PEAK_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload),
             "kernel": "gemm_kernel", "avg_launch_ms": round(ms_per_step / launches, 5),
             "flops_per_launch": flops_per_step / launches, "algorithmic_bytes_per_launch": bytes_per_step / launches,
         },
