@@ -70,6 +70,23 @@ CASES = [
     (GemmConfig(128, 128, 16, 64, 64, 32, 2, 0, 0, 4, 1), [(200, 300, 72)]),           # unpadded LDS
     (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 4, 4, 1), [(200, 300, 72)]),           # padded LDS-B
 ]
+# pipeline depth 3 (register stage + split last round): every path of its step driver -- an even and an
+# odd number of fragment rounds per K step, 1, 2, 3, 4 and many K steps, ragged K, every operand width
+CASES += [
+    (GemmConfig(128, 128, 32, 64, 64, 32, 3, 4, 0, 4, 1), [(200, 300, 32), (200, 300, 64), (130, 260, 96), (200, 300, 200)]),
+    (GemmConfig(128, 128, 8, 64, 64, 32, 3, 4, 0, 4, 1), [(140, 132, 8), (140, 132, 16), (140, 132, 24), (140, 132, 32), (140, 132, 72), (140, 132, 100)]),
+    (GemmConfig(128, 128, 24, 64, 64, 32, 3, 4, 0, 4, 1), [(140, 132, 24), (140, 132, 48), (140, 132, 120), (140, 132, 100)]),
+    (GemmConfig(128, 128, 16, 64, 64, 16, 3, 4, 0, 4, 1), [(200, 300, 16), (200, 300, 48), (33, 36, 80)]),
+    (GemmConfig(128, 128, 32, 32, 64, 32, 3, 4, 0, 4, 0), [(256, 384, 128)]),
+    (GemmConfig(128, 128, 64, 32, 64, 16, 3, 4, 0, 4, 1), [(200, 300, 136)]),
+    (GemmConfig(256, 256, 32, 64, 128, 32, 3, 4, 0, 4, 1), [(512, 768, 160), (300, 520, 100)]),
+    (GemmConfig(256, 256, 32, 128, 128, 32, 3, 4, 0, 4, 0), [(512, 512, 64)]),
+    (GemmConfig(256, 128, 32, 64, 64, 32, 3, 4, 0, 4, 1), [(300, 260, 100)]),
+    (GemmConfig(128, 128, 16, 64, 64, 32, 3, 4, 0, 1, 1), [(37, 53, 29), (130, 127, 17)]),
+    (GemmConfig(32, 64, 8, 32, 32, 32, 3, 4, 0, 4, 1), [(70, 92, 52)]),          # fewer load units than threads
+    (GemmConfig(64, 64, 16, 16, 64, 16, 3, 4, 0, 1, 1), [(70, 90, 50)]),
+    (GemmConfig(128, 128, 32, 64, 32, 32, 3, 4, 0, 4, 1), [(200, 300, 72)]),      # one column block per wave
+]
 FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
 
 
@@ -107,7 +124,8 @@ def test_accumulate_mode_adds_into_c(device):
     C0 = np.random.default_rng(12).integers(-50, 50, (M, N)).astype(np.float32)
     for cfg in (GemmConfig(256, 128, 32, 64, 128, 32, 2, 4, 0, 4, 1, 3, 8, 1),
                 GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 1, 1, 3, 8, 1),
-                GemmConfig(128, 128, 16, 64, 32, 32, 2, 4, 0, 4, 1, 3, 8, 1)):
+                GemmConfig(128, 128, 16, 64, 32, 32, 2, 4, 0, 4, 1, 3, 8, 1),
+                GemmConfig(128, 128, 32, 32, 64, 32, 3, 4, 0, 4, 1, 3, 8, 1)):
         got = run_gemm(cfg, A, B, c_init=C0)
         assert np.array_equal(got, go.c_gemm_f32(A, B, out=C0.copy(), accumulate=True)), cfg.tag()
 
@@ -172,6 +190,15 @@ def test_results_are_bitwise_reproducible_and_independent_of_tile_order(device):
     assert np.array_equal(first, run_gemm(GemmConfig(128, 128, 32, 64, 64, 32, 2, 4, 0, 4, 1), A, B))
 
 
+def test_pipeline_depth_does_not_change_the_bits(device):
+    """Depths 1, 2 and 3 schedule the same MFMAs in the same order per accumulator."""
+    M, N, K = 384, 512, 416
+    A, B = go.make_inputs(M, N, K, seed=41)
+    for bk, mi in ((32, 32), (16, 16), (8, 32)):
+        outs = [run_gemm(GemmConfig(128, 128, bk, 64, 64, mi, stages, 4, 0, 4, 1), A, B) for stages in (1, 2, 3)]
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[2]), (bk, mi)
+
+
 def test_plan_cache_and_one_shot_entry_point(device):
     cfg = GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 1)
     p1, p2 = GemmPlan(cfg), GemmPlan(cfg)
@@ -226,7 +253,7 @@ def test_named_configs_full_size_through_policy_and_compiler(device, name, shape
     dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B)
     for hint in hints:
         say(name, hint)
-        func = roller.Compiler(cfg, hint, 2, dump_path=tmp_path if hint is hints[0] else None).compile()
+        func = roller.Compiler(cfg, hint, bm.PIPELINE_DEPTH, dump_path=tmp_path if hint is hints[0] else None).compile()
         dC = DeviceArray((shape[0], shape[1]))
         dC.fill_bytes(0xFF)
         func(func.grid_dims(), func.block_dims(), (dA.ptr, dB.ptr, dC.ptr), shared_mem=hint.smem_cost * 2)
@@ -249,7 +276,7 @@ def test_m0_to_m13_exact_on_integer_inputs_at_full_size(device):
         hint = get_roller_hints(cfg, arch, topk=1)[0]
         say(f"M{i}", shape, hint.block_tile, hint.wave_tile, hint.rstep)
         A, B = go.make_inputs(*shape, seed=i, distribution="integer")
-        func = roller.Compiler(cfg, hint).compile()
+        func = roller.Compiler(cfg, hint, bm.PIPELINE_DEPTH).compile()
         dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray((shape[0], shape[1]))
         func(func.grid_dims(), func.block_dims(), (dA, dB, dC))
         hip.synchronize()
@@ -273,8 +300,8 @@ def test_handle_checks_grid_and_block(device):
 def test_run_eval_and_sweep_end_to_end(device, tmp_path, capsys):
     cfg = MatmulConfig(1024, 1024, 512, 32)
     hint = get_roller_hints(cfg, MI355X.from_device(device), topk=1)[0]
-    func = roller.Compiler(cfg, hint, 2).compile()
-    ms, gflops = roller.run_eval(func, 2, hint, repeat_times=5)
+    func = roller.Compiler(cfg, hint, 3).compile()
+    ms, gflops = roller.run_eval(func, 3, hint, repeat_times=5)
     assert ms > 0 and gflops == pytest.approx(2 * 1024 * 1024 * 512 * 1e-9 / (ms / 1e3), rel=1e-6)
     assert func.last_eval["ok"] and func.last_eval["normwise"] <= 1e-5
     df = bm.benchmark([(512, 768, 256), (300, 500, 96)], topk=4, csv_path=tmp_path / "r.csv", repeat_times=3)
