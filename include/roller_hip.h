@@ -69,6 +69,8 @@ typedef struct rl_gemm_config {
   int swz;         /* bit0: XCD-contiguous tile order, bit1: panel walk              */
   int group;       /* panel height in tiles (reference: panel-width=8, roller.py:338)*/
   int accum;       /* 0: C = A*B, 1: C += A*B (linalg.matmul semantics, roller.py:62)*/
+  int direct;      /* 1: global loads write LDS directly (no staging registers, swizzled
+                      A rows); needs stages=3, vec=4, pad_a=pad_b=0, bk a power of 2 */
 } rl_gemm_config;
 
 /* ---- library / device ---------------------------------------------------------------------- */

@@ -339,9 +339,14 @@ class Policy:
 
     def _expand_reduce_axis(self, td: TileDict) -> None:
         """Grows ``td.rstep`` to the multiple of the base step that gives the longest contiguous
-        operand rows while one stage still fits the block's share of workgroup memory.  Only
+        operand rows while one stage still fits the block's share of workgroup memory (the
+        share among the blocks a core actually hosts, when matrix cores are modelled).  Only
         ``rstep`` and ``smem_cost`` change; occupancy figures keep their base-step values."""
-        limit = min(self.arch.max_smem_usage // td.block_per_SM, self.arch.smem_cap)
+        resident = td.block_per_SM
+        if self.arch.has_matrix_cores:
+            # a grid that does not fill the device leaves each core fewer blocks to host
+            resident = max(1, min(resident, -(-td.grid_size // self.arch.compute_max_core)))
+        limit = min(self.arch.max_smem_usage // resident, self.arch.smem_cap)
         steps = [
             s for s in self.get_reduce_step_candidates(self.matmul_config.K)
             if s % td.rstep == 0 and td.infer_smem_usage(s) <= limit

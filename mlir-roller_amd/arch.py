@@ -107,9 +107,8 @@ class MI355X(TileDevice):
     reg_estimate_divisor: int = 4
     # 256 accumulation registers per lane are available next to the architectural ones
     thread_reg_limit: int = 257
-    # rows of the LDS A tile are padded by one 16-byte unit so that 128-bit reads of
-    # consecutive rows fall into distinct bank groups
-    lds_row_pad: int = 4
+    # the kernel's direct-to-LDS path swizzles the A rows instead of padding them
+    lds_row_pad: int = 0
     # two waves per SIMD let one wave's LDS traffic and barriers hide behind the other's MFMAs
     waves_per_partition: int = 2
     # 256 architectural + 256 accumulation registers per lane, shared by the waves of a SIMD

@@ -31,6 +31,13 @@
 //               bit1 = walk the tile grid in panels of GROUP tile rows
 //   GROUP, NXCD panel height in tiles; number of XCDs the dispatcher round-robins over
 //   ACCUM       1 = C += A*B (what linalg.matmul means, roller.py:62), 0 = C = A*B
+//   DIRECT      1 = global loads write LDS directly (buffer_load_dwordx4 ... lds), no staging
+//               registers and no LDS write instructions; needs STAGES=3, VEC=4, PAD_A=PAD_B=0
+//               and BK a power of two.
+//               A wave's load lands as 64 consecutive 16-byte units, so rows cannot be padded;
+//               instead the 16-byte chunks of every A row are XOR-swizzled with the row number
+//               (on the load side by choosing which global chunk a lane fetches, on the read
+//               side in the fragment address), which keeps the 128-bit A reads conflict-free.
 //
 // Layout trick that removes every LDS bank conflict and every register shuffle on the read side:
 // an MFMA sums over its k slots, and a GEMM does not care which MFMA block owns which column, so
@@ -101,6 +108,9 @@
 #ifndef SCHED
 #define SCHED 1
 #endif
+#ifndef DIRECT
+#define DIRECT 0
+#endif
 
 #define NWM (BM / WM)
 #define NWN (BN / WN)
@@ -124,6 +134,10 @@
 #define A_PER_T ((A_UNITS + NT - 1) / NT)
 #define B_PER_T ((B_UNITS + NT - 1) / NT)
 #define OOB_OFFSET 0x80000000u
+/* DIRECT: 16-byte chunks per A row, A rows per 128 bytes of LDS, and the swizzle period */
+#define CPR (BK / 4)
+#define RPL (CPR >= 8 ? 1 : 8 / CPR)
+#define SWZ_N (CPR >= 8 ? 8 : CPR)
 
 static_assert(MI == 32 || MI == 16, "MI selects v_mfma_f32_32x32x2_f32 or v_mfma_f32_16x16x4_f32");
 static_assert(BM % WM == 0 && BN % WN == 0, "wave tile must divide block tile");
@@ -134,6 +148,9 @@ static_assert(PAD_A % 4 == 0 && PAD_B % 4 == 0, "LDS rows stay 16-byte aligned")
 static_assert(NT <= 1024, "at most 16 waves per workgroup");
 static_assert(STAGES >= 1 && STAGES <= 3, "pipeline depth 1, 2 or 3");
 static_assert(VEC == 4 || VEC == 1, "global access width");
+static_assert(!DIRECT || (STAGES == 3 && VEC == 4 && PAD_A == 0 && PAD_B == 0), "DIRECT needs STAGES=3, VEC=4, no padding");
+static_assert(!DIRECT || (A_UNITS % 64 == 0 && B_UNITS % 64 == 0), "DIRECT moves whole waves of 16-byte units");
+static_assert(!DIRECT || (BK & (BK - 1)) == 0, "DIRECT swizzles A rows with XOR: BK must be a power of two");
 static_assert(LDS_BUFS * STAGE_FLOATS * 4 <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
 
 typedef float v2f __attribute__((ext_vector_type(2)));
@@ -272,7 +289,12 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
   for (int i = 0; i < A_PER_T; ++i) {
     const int u = tid + i * NT;
+#if DIRECT
+    // LDS unit u of the tile is (row, slot u % CPR); it holds chunk slot ^ swizzle(row) of that row
+    const int row = u / CPR, c = (u % CPR) ^ ((row / RPL) % SWZ_N);
+#else
     const int row = u / (BK / 4), c = u % (BK / 4);
+#endif
     a_goff[i] = (unsigned)(row * lda + c * 4) * 4u;
     a_soff[i] = row * LDA_S + c * 4;
     a_kcol[i] = c * 4;
@@ -295,9 +317,41 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   long a_rem = ((long)(M - m0 - 1) * lda + K) * 4;        // valid bytes from Ag to the end of A
   long b_rem = ((long)(K - 1) * ldb + (N - n0)) * 4;      // valid bytes from Bg to the end of B
 
+#if !DIRECT
   v4f ra[A_PER_T], rb[B_PER_T];
+#endif
 
   const int KT = (K + BK - 1) / BK;
+
+#if DIRECT
+  // Issues the loads of K step kt straight into LDS buffer `stage`.  Instruction i of a wave
+  // fills the 64 consecutive 16-byte units that start at unit i*NT + wave*64 of the operand tile.
+  auto fetch_direct = [&](int kt, int stage) {
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+    const int k0 = kt * BK;
+    const bool live = kt < KT;
+    const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, live ? a_rem - (long)k0 * 4 : 0);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + (long)k0 * ldb, live ? b_rem - (long)k0 * ldb * 4 : 0);
+    float* As = lds + stage * STAGE_FLOATS;
+    float* Bs = As + A_STAGE;
+#pragma unroll
+    for (int i = 0; i < A_PER_T; ++i) {
+      const int first = i * NT + wave * 64;
+      if (A_UNITS % NT == 0 || first < A_UNITS) {
+        const bool ok = a_ok[i] && (!EDGE || k0 + a_kcol[i] < K);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr_t)(As + first * 4), 16, ok ? a_goff[i] : OOB_OFFSET, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < B_PER_T; ++i) {
+      const int first = i * NT + wave * 64;
+      if (B_UNITS % NT == 0 || first < B_UNITS) {
+        const bool ok = b_ok[i][0] && (!EDGE || k0 + b_krow[i] < K);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(br, (lds_ptr_t)(Bs + first * 4), 16, ok ? b_goff[i] : OOB_OFFSET, 0, 0, 0);
+      }
+    }
+  };
+#else
 
   // Issues the global loads of K step kt into the staging registers.  A step at or beyond KT
   // (the pipelined loop asks for up to two steps ahead) gets an empty resource: every load
@@ -332,6 +386,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < B_PER_T; ++i)
       if (B_UNITS % NT == 0 || tid + i * NT < B_UNITS) *(v4f*)&Bs[b_soff[i]] = rb[i];
   };
+#endif
 
   acc_t acc[TM][TN];
 #pragma unroll
@@ -341,7 +396,14 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
       for (int r = 0; r < ACC_REGS; ++r) acc[i][j][r] = 0.0f;
 
+#if DIRECT
+  const int a_frag = (wm0 + lr) * LDA_S;            // + bi*MI*LDA_S + swizzled chunk of the round
+  int a_round[SUPERS];
+#pragma unroll
+  for (int r = 0; r < SUPERS; ++r) a_round[r] = ((r * (KSUPER / 4) + lg) ^ ((lr / RPL) % SWZ_N)) * 4;
+#else
   const int a_frag = (wm0 + lr) * LDA_S + 4 * lg;   // + bi*MI*LDA_S + kk
+#endif
   const int b_frag = (4 * lg) * LDB_S + wn0 + VN * lr;  // + (kk+t)*LDB_S + v*MI*VN
 
   // One round of LDS fragment reads: TM 128-bit reads of A (four consecutive k each) and, for each
@@ -354,7 +416,11 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const float* As = lds + stage * STAGE_FLOATS;
     const float* Bs = As + A_STAGE;
 #pragma unroll
+#if DIRECT
+    for (int bi = 0; bi < TM; ++bi) f.a[bi] = *(const v4f*)&As[a_frag + bi * MI * LDA_S + a_round[kk / KSUPER]];
+#else
     for (int bi = 0; bi < TM; ++bi) f.a[bi] = *(const v4f*)&As[a_frag + bi * MI * LDA_S + kk];
+#endif
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
@@ -386,9 +452,15 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // loads of tile kt+2 are issued, the workgroup meets at the barrier, and the first fragment
     // round of tile kt+1 is read -- so that the last MFMA group covers that read's latency.
     frag_t fr[2];
+#if DIRECT
+    fetch_direct(0, 0);
+    fetch_direct(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of both tiles is in LDS
+#else
     fetch(0);
     stash(0);
     fetch(1);
+#endif
     __syncthreads();
     read_frags(fr[0], 0, 0);
 
@@ -408,6 +480,23 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       // the last round is split around the barrier: its first half covers the LDS writes of
       // tile kt+1 and the global loads of tile kt+2, its second half the first reads of tile kt+1
       mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
+#if DIRECT
+      // Tile kt+1 was requested one step ago, straight into the other buffer; once every wave's
+      // part has landed and all have met, buffer `cur` is free again and takes tile kt+2.
+#if SCHED
+#pragma unroll
+      for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
+#endif
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      __syncthreads();
+      read_frags(fr[(P + SUPERS) & 1], cur ^ 1, 0);
+      fetch_direct(kt + 2, cur);
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 2, 4);
+#if SCHED
+      interleave_with_mfma<G / 4, R, 0x100>();
+      interleave_with_mfma<G / 2 - G / 4, L, 0x020>();
+#endif
+#else
       stash(cur ^ 1);
       fetch(kt + 2);
 #if SCHED
@@ -422,6 +511,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #if SCHED
       interleave_with_mfma<G / 2, R, 0x100>();
 #endif
+#endif
     };
     auto last_step = [&](auto parity, int kt) {
       constexpr int P = decltype(parity)::value;
@@ -435,6 +525,9 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #if SCHED
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
+#endif
+#if DIRECT
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // the (empty) request for the tile past the end has drained
 #endif
     };
 
@@ -457,6 +550,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     }
   }
 #else
+  static_assert(!DIRECT, "DIRECT belongs to the pipelined loop");
   auto multiply = [&](int stage) {
 #pragma unroll
     for (int kk = 0; kk < BK; kk += KSUPER) {

@@ -116,6 +116,14 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
   if ((c.edge | 1) != 1 || (c.accum | 1) != 1) return fail(RL_ERR_INVALID_ARG, "edge and accum are 0 or 1");
   if (c.swz < 0 || c.swz > 3) return fail(RL_ERR_INVALID_ARG, "swz is a 2-bit mask");
   if ((c.swz & 2) && c.group <= 0) return fail(RL_ERR_INVALID_ARG, "group must be positive");
+  if ((c.direct | 1) != 1) return fail(RL_ERR_INVALID_ARG, "direct is 0 or 1");
+  if (c.direct) {
+    if (c.stages != 3 || c.vec != 4 || c.pad_a || c.pad_b)
+      return fail(RL_ERR_INVALID_ARG, "direct=1 needs stages=3, vec=4, pad_a=0, pad_b=0");
+    if (c.bk & (c.bk - 1)) return fail(RL_ERR_INVALID_ARG, "direct=1 needs bk to be a power of two (XOR swizzle), got %d", c.bk);
+    if ((c.bm * c.bk / 4) % 64 || (c.bk * c.bn / 4) % 64)
+      return fail(RL_ERR_INVALID_ARG, "direct=1 needs bm*bk and bk*bn to be multiples of 256 (whole waves of 16-byte units)");
+  }
   const int nt = 64 * (c.bm / c.wm) * (c.bn / c.wn);
   if (nt > 1024) return fail(RL_ERR_INVALID_ARG, "%d threads per workgroup exceed 1024", nt);
   const long lds = (long)(c.stages >= 2 ? 2 : 1) * ((long)c.bm * (c.bk + c.pad_a) + (long)c.bk * (c.bn + c.pad_b)) * 4;
@@ -131,6 +139,7 @@ std::vector<std::string> config_options(const rl_gemm_config& c) {
   def("BM", c.bm); def("BN", c.bn); def("BK", c.bk); def("WM", c.wm); def("WN", c.wn); def("MI", c.mi);
   def("STAGES", c.stages); def("PAD_A", c.pad_a); def("PAD_B", c.pad_b); def("VEC", c.vec);
   def("EDGE", c.edge); def("SWZ", c.swz); def("GROUP", c.group > 0 ? c.group : 1); def("ACCUM", c.accum);
+  def("DIRECT", c.direct);
   return o;
 }
 

@@ -61,7 +61,7 @@ class DeviceProps(C.Structure):
 class _GemmConfigC(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "bm", "bn", "bk", "wm", "wn", "mi", "stages", "pad_a", "pad_b", "vec", "edge", "swz",
-        "group", "accum")]
+        "group", "accum", "direct")]
 
 
 @dataclass(frozen=True)
@@ -82,6 +82,7 @@ class GemmConfig:
     swz: int = 3
     group: int = 8
     accum: int = 0
+    direct: int = 0
 
     def to_c(self) -> _GemmConfigC:
         return _GemmConfigC(*(getattr(self, f.name) for f in fields(self)))
@@ -97,7 +98,7 @@ class GemmConfig:
     def tag(self) -> str:
         return (f"b{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_mi{self.mi}_s{self.stages}"
                 f"_p{self.pad_a}.{self.pad_b}_v{self.vec}_e{self.edge}_z{self.swz}.{self.group}"
-                f"_a{self.accum}")
+                f"_a{self.accum}" + ("_d1" if self.direct else ""))
 
 
 # --------------------------------------------------------------------------------------------

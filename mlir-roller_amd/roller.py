@@ -60,14 +60,19 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
                              f"for {threads} threads and reduce step {bk}")
         (wm, wn), mi = split
     M, N, K = config.M, config.N, config.K
-    # (bk + pad)/4 odd keeps the 128-bit reads of LDS-A free of bank conflicts
-    pad_a = 4 if (bk // 4) % 2 == 0 else 0
+    stages = max(1, min(3, int(pipeline_depth)))
+    vec = 4 if (K % 4 == 0 and N % 4 == 0) else 1
+    # At full depth and width the global loads go straight to LDS (swizzled A rows, no padding)
+    # whenever both operand tiles are whole waves of 16-byte units and the K step is a power of
+    # two (the swizzle is an XOR).
+    direct = int(stages == 3 and vec == 4 and bk & (bk - 1) == 0
+                 and (bm * bk // 4) % 64 == 0 and (bk * bn // 4) % 64 == 0)
+    # otherwise (bk + pad)/4 odd keeps the 128-bit reads of LDS-A free of bank conflicts
+    pad_a = 0 if direct else (4 if (bk // 4) % 2 == 0 else 0)
     return GemmConfig(
-        bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi,
-        stages=max(1, min(3, int(pipeline_depth))), pad_a=pad_a, pad_b=0,
-        vec=4 if (K % 4 == 0 and N % 4 == 0) else 1,
+        bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi, stages=stages, pad_a=pad_a, pad_b=0, vec=vec,
         edge=0 if (M % bm == 0 and N % bn == 0 and K % bk == 0) else 1,
-        swz=3, group=8, accum=1 if accumulate else 0,
+        swz=3, group=8, accum=1 if accumulate else 0, direct=direct,
     )
 
 

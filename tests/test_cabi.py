@@ -59,6 +59,10 @@ def test_config_check_accepts_and_sizes(hip_lib):
     (dict(bm=1024, bn=1024, wm=32, wn=32, bk=8), "threads per workgroup"),
     (dict(edge=2), "edge and accum"),
     (dict(mi=16, bk=8), "bk must be a multiple of 16"),
+    (dict(direct=1), "direct=1 needs stages=3"),
+    (dict(direct=1, stages=3, pad_a=0, vec=1), "direct=1 needs stages=3"),
+    (dict(direct=2), "direct is 0 or 1"),
+    (dict(direct=1, stages=3, pad_a=0, bk=24), "power of two"),
 ])
 def test_config_check_rejects(hip_lib, bad, needle):
     with pytest.raises(HipError) as err:

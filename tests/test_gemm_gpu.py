@@ -87,6 +87,21 @@ CASES += [
     (GemmConfig(64, 64, 16, 16, 64, 16, 3, 4, 0, 1, 1), [(70, 90, 50)]),
     (GemmConfig(128, 128, 32, 64, 32, 32, 3, 4, 0, 4, 1), [(200, 300, 72)]),      # one column block per wave
 ]
+# direct-to-LDS loads with swizzled A rows: every swizzle period (K step 8, 16, 32, 64), both MFMA shapes,
+# ragged edges in all three dimensions (out-of-range lanes must deposit zeros), 1..many K steps
+CASES += [
+    (GemmConfig(128, 128, 32, 32, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 300, 32), (200, 300, 64), (130, 260, 96), (200, 300, 200), (1, 4, 4)]),
+    (GemmConfig(128, 128, 8, 64, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(140, 132, 8), (140, 132, 16), (140, 132, 24), (140, 132, 100)]),
+    (GemmConfig(128, 128, 16, 64, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(140, 132, 48), (140, 132, 100)]),
+    (GemmConfig(128, 128, 64, 32, 64, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 300, 136), (128, 128, 64)]),
+    (GemmConfig(128, 128, 16, 64, 64, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 300, 16), (33, 36, 80)]),
+    (GemmConfig(256, 256, 32, 64, 128, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(512, 768, 160), (300, 520, 100)]),
+    (GemmConfig(256, 256, 32, 128, 128, 32, 3, 0, 0, 4, 0, 3, 8, 0, 1), [(512, 512, 64)]),
+    (GemmConfig(256, 128, 32, 64, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(300, 260, 100)]),
+    (GemmConfig(32, 64, 8, 32, 32, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(70, 92, 52)]),       # fewer load units than threads
+    (GemmConfig(64, 64, 16, 16, 64, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(70, 92, 52)]),
+    (GemmConfig(128, 128, 32, 64, 32, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 300, 72)]),
+]
 FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
 
 
@@ -125,7 +140,8 @@ def test_accumulate_mode_adds_into_c(device):
     for cfg in (GemmConfig(256, 128, 32, 64, 128, 32, 2, 4, 0, 4, 1, 3, 8, 1),
                 GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 1, 1, 3, 8, 1),
                 GemmConfig(128, 128, 16, 64, 32, 32, 2, 4, 0, 4, 1, 3, 8, 1),
-                GemmConfig(128, 128, 32, 32, 64, 32, 3, 4, 0, 4, 1, 3, 8, 1)):
+                GemmConfig(128, 128, 32, 32, 64, 32, 3, 4, 0, 4, 1, 3, 8, 1),
+                GemmConfig(128, 128, 32, 32, 64, 32, 3, 0, 0, 4, 1, 3, 8, 1, 1)):
         got = run_gemm(cfg, A, B, c_init=C0)
         assert np.array_equal(got, go.c_gemm_f32(A, B, out=C0.copy(), accumulate=True)), cfg.tag()
 
@@ -191,12 +207,14 @@ def test_results_are_bitwise_reproducible_and_independent_of_tile_order(device):
 
 
 def test_pipeline_depth_does_not_change_the_bits(device):
-    """Depths 1, 2 and 3 schedule the same MFMAs in the same order per accumulator."""
+    """Depths 1, 2, 3 and the direct-to-LDS variant run the same MFMAs in the same order per
+    accumulator; only the way operands reach LDS differs."""
     M, N, K = 384, 512, 416
     A, B = go.make_inputs(M, N, K, seed=41)
     for bk, mi in ((32, 32), (16, 16), (8, 32)):
         outs = [run_gemm(GemmConfig(128, 128, bk, 64, 64, mi, stages, 4, 0, 4, 1), A, B) for stages in (1, 2, 3)]
-        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[1], outs[2]), (bk, mi)
+        outs.append(run_gemm(GemmConfig(128, 128, bk, 64, 64, mi, 3, 0, 0, 4, 1, 3, 8, 0, 1), A, B))   # direct-to-LDS
+        assert all(np.array_equal(outs[0], o) for o in outs[1:]), (bk, mi)
 
 
 def test_plan_cache_and_one_shot_entry_point(device):

@@ -17,14 +17,26 @@ def test_hint_to_gemm_config_aligned_problem():
     hint = next(h for h in get_roller_hints(cfg, MI355X(), 20) if h.block_tile == [256, 256])
     g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=2)
     assert (g.bm, g.bn, g.bk, g.wm, g.wn, g.mi) == (256, 256, hint.rstep, *hint.wave_tile, hint.mfma)
-    assert (g.stages, g.vec, g.edge, g.accum) == (2, 4, 0, 0)
+    assert (g.stages, g.vec, g.edge, g.accum, g.direct) == (2, 4, 0, 0, 0)
     assert ((g.bk + g.pad_a) // 4) % 2 == 1          # odd number of 16-byte units per LDS-A row
+    g3 = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3)
+    assert (g3.stages, g3.direct, g3.pad_a, g3.pad_b) == (3, 1, 0, 0)   # direct-to-LDS: swizzle instead of padding
     assert g.threads == hint.threads and g.lds_bytes <= 160 * 1024
     assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=1).stages == 1
     assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).stages == 3
     assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=5).stages == 3
-    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).lds_bytes == g.lds_bytes   # still two LDS buffers
+    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).lds_bytes == 2 * hint.smem_cost   # still two LDS buffers
     assert roller.hint_to_gemm_config(cfg, hint, accumulate=True).accum == 1
+
+
+def test_direct_path_needs_a_power_of_two_k_step():
+    cfg = MatmulConfig(1536, 1536, 1536, 32)
+    hint = get_roller_hints(cfg, MI355X(), 1)[0].clone()
+    hint.rstep = 48
+    g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3)
+    assert (g.bk, g.direct, g.pad_a) == (48, 0, 4)
+    hint.rstep = 64
+    assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).direct == 1
 
 
 def test_hint_to_gemm_config_ragged_problem():
@@ -32,8 +44,8 @@ def test_hint_to_gemm_config_ragged_problem():
     g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0])
     assert g.edge == 1 and g.vec == 4                # 5000 and 1536 are multiples of 4
     cfg = MatmulConfig(37, 53, 29, 32)
-    g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0])
-    assert g.edge == 1 and g.vec == 1
+    g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0], pipeline_depth=3)
+    assert g.edge == 1 and g.vec == 1 and g.direct == 0 and g.pad_a == 4   # dword path keeps padded rows
 
 
 def test_hint_from_the_a100_model_still_maps_to_wave_tiles():

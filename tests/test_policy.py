@@ -235,10 +235,10 @@ def test_mi355x_hints_are_launchable_kernel_configs(shape):
         dims = utils.get_block_dims(h.block_tile + [0], h.thread_tile + [0])
         assert dims[0] * dims[1] == h.threads
         assert h.thread_tile[0] * h.thread_tile[1] <= 256          # accumulators per lane
-        assert h.smem_cost == (h.rstep * (m + n) + 4 * m) * 4         # one stage, LDS-A rows padded
+        assert h.smem_cost == h.rstep * (m + n) * 4                   # one stage, rows unpadded (swizzled)
         assert 2 * h.smem_cost <= arch.lds_bytes                    # double-buffered tile fits a CU
-        g = hint_to_gemm_config(cfg, h, 2)
-        assert g.lds_bytes == 2 * h.smem_cost
+        g = hint_to_gemm_config(cfg, h, 3)
+        assert g.lds_bytes == 2 * h.smem_cost or g.direct == 0    # padded rows only on the dword path
         assert h.grid_size == math.ceil(cfg.M / m) * math.ceil(cfg.N / n)
 
 
@@ -304,3 +304,16 @@ def test_mi355x_register_budget_drops_splits_that_would_spill():
     assert [h.threads for h in policy._assign_wave_tiles(td, 512)] == [512, 512]   # 128 + 96 <= 256
     assert policy._assign_wave_tiles(td, 1024) == []                               # 64 + 96 > 128
     assert policy._assign_wave_tiles(td, 96) == []                                 # not a whole number of waves
+
+
+def test_mi355x_reduce_step_grows_when_the_grid_leaves_room():
+    arch = MI355X()
+    # 2048^2 output, 128x128 tiles: 256 blocks on 256 CUs -> one block per CU -> the whole 80 KB stage budget
+    small = get_roller_hints(MatmulConfig(2048, 2048, 2048, 32), arch, topk=1)[0]
+    assert (small.block_tile, small.rstep, small.smem_cost) == ([128, 128], 64, 65536)
+    # 4096x8192 output with the same tile: 8 blocks per CU, two resident -> 40 KB each -> step stays 32
+    cfg = MatmulConfig(4096, 8192, 4096, 32)
+    policy = Policy(cfg, arch)
+    td = TileDict.from_block_tile([128, 128], 32, cfg, arch)
+    policy._expand_reduce_axis(td)
+    assert td.rstep == 32
