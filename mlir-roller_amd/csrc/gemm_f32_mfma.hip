@@ -134,10 +134,14 @@
 #define A_PER_T ((A_UNITS + NT - 1) / NT)
 #define B_PER_T ((B_UNITS + NT - 1) / NT)
 #define OOB_OFFSET 0x80000000u
-/* DIRECT: 16-byte chunks per A row, A rows per 128 bytes of LDS, and the swizzle period */
+/* DIRECT: 16-byte chunks per A row; A rows per 256 bytes of LDS (the 64 banks that a 128-bit read
+ * of 16 lanes must cover without collision); the swizzle period.  Rows that start at the same
+ * offset within a 256-byte window get their chunks XOR-ed with distinct values, so the 16 lanes
+ * of one read cycle, which sit in 16 consecutive rows at the same chunk, hit 16 distinct bank
+ * groups. */
 #define CPR (BK / 4)
-#define RPL (CPR >= 8 ? 1 : 8 / CPR)
-#define SWZ_N (CPR >= 8 ? 8 : CPR)
+#define RPL (CPR >= 16 ? 1 : 16 / CPR)
+#define SWZ_N (CPR >= 16 ? 16 : CPR)
 
 static_assert(MI == 32 || MI == 16, "MI selects v_mfma_f32_32x32x2_f32 or v_mfma_f32_16x16x4_f32");
 static_assert(BM % WM == 0 && BN % WN == 0, "wave tile must divide block tile");
