@@ -155,8 +155,12 @@ class TileDict:
     def infer_smem_usage(self, rstep: Optional[int] = None) -> int:
         """Bytes of workgroup memory for one pipeline stage: an [m, rstep] and an [rstep, n] tile."""
         step = self.rstep if rstep is None else rstep
-        # the kernel pads every row of the [m, rstep] tile by ``lds_row_pad`` elements
-        return (step * sum(self.block_tile) + self.lds_row_pad * self.block_tile[0]) * self.matmul_config.el_bytes
+        cfg = self.matmul_config
+        # The MFMA kernel keeps the [m, rstep] tile unpadded only on its direct-to-LDS path: K and N
+        # multiples of 4 and a power-of-two step.  Otherwise every row grows by ``lds_row_pad``.
+        swizzled = cfg.K % 4 == 0 and cfg.N % 4 == 0 and step & (step - 1) == 0
+        pad = 0 if swizzled else self.lds_row_pad
+        return (step * sum(self.block_tile) + pad * self.block_tile[0]) * cfg.el_bytes
 
     @classmethod
     def from_block_tile(cls, block_tile: List[int], rstep: int, matmul_config: MatmulConfig,

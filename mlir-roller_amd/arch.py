@@ -37,6 +37,7 @@ class TileDevice:
     # a per-lane accumulator tile needing this many 32-bit registers or more is rejected
     thread_reg_limit: int = 256
     # elements of padding the kernel adds to every row of the [m, rstep] workgroup-memory tile
+    # when it cannot use its unpadded (swizzled) layout
     lds_row_pad: int = 0
     # warps per scheduler that the block-size recommendation aims for
     waves_per_partition: int = 1
@@ -107,8 +108,9 @@ class MI355X(TileDevice):
     reg_estimate_divisor: int = 4
     # 256 accumulation registers per lane are available next to the architectural ones
     thread_reg_limit: int = 257
-    # the kernel's direct-to-LDS path swizzles the A rows instead of padding them
-    lds_row_pad: int = 0
+    # the kernel's register-staged path pads every row of the LDS A tile by one 16-byte unit; its
+    # direct-to-LDS path (K, N multiples of 4 and a power-of-two reduce step) swizzles instead
+    lds_row_pad: int = 4
     # two waves per SIMD let one wave's LDS traffic and barriers hide behind the other's MFMAs
     waves_per_partition: int = 2
     # 256 architectural + 256 accumulation registers per lane, shared by the waves of a SIMD

@@ -273,8 +273,11 @@ int opt_in_lds(hipFunction_t f, int bytes) {
   return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
 }
 
+// The current device is a per-thread setting of the HIP runtime; a thread other than the one that
+// called rl_init would otherwise work on device 0.
 int ensure_ready() {
   if (!g_ready) return fail(RL_ERR_NO_DEVICE, "rl_init has not been called (or failed)");
+  HIP_TRY(hipSetDevice(g_device));
   return RL_OK;
 }
 

@@ -235,10 +235,11 @@ def test_mi355x_hints_are_launchable_kernel_configs(shape):
         dims = utils.get_block_dims(h.block_tile + [0], h.thread_tile + [0])
         assert dims[0] * dims[1] == h.threads
         assert h.thread_tile[0] * h.thread_tile[1] <= 256          # accumulators per lane
-        assert h.smem_cost == h.rstep * (m + n) * 4                   # one stage, rows unpadded (swizzled)
+        swizzled = cfg.K % 4 == 0 and cfg.N % 4 == 0 and h.rstep & (h.rstep - 1) == 0
+        assert h.smem_cost == (h.rstep * (m + n) + (0 if swizzled else 4 * m)) * 4   # one stage; padded rows off the direct path
         assert 2 * h.smem_cost <= arch.lds_bytes                    # double-buffered tile fits a CU
         g = hint_to_gemm_config(cfg, h, 3)
-        assert g.lds_bytes == 2 * h.smem_cost or g.direct == 0    # padded rows only on the dword path
+        assert g.lds_bytes == 2 * h.smem_cost and g.direct == int(swizzled)
         assert h.grid_size == math.ceil(cfg.M / m) * math.ceil(cfg.N / n)
 
 
