@@ -131,6 +131,33 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
     return df
 
 
+def plot_results(df: pd.DataFrame, path: os.PathLike, peak_tflops: float = 157.3) -> Path:
+    """Bar chart of the sweep, one bar per shape labelled M0, M1, ... like the reference's
+    ``images/gemm_fp32_benchmark.png`` (README.md:4-9).  The reference plots speedup over
+    cuBLAS; with no vendor-BLAS column here the bars show % of the fp32-matrix peak, and the
+    host baseline appears as the speedup printed above each bar."""
+    import matplotlib
+    matplotlib.use("Agg")
+    import matplotlib.pyplot as plt
+
+    labels = [f"M{i}" for i in range(len(df))]
+    pct = 100.0 * df["Roller TFLOPS"] / peak_tflops
+    fig, ax = plt.subplots(figsize=(max(6.0, 0.6 * len(df) + 2.0), 4.0))
+    bars = ax.bar(labels, pct, color="#c8102e")
+    ax.axhline(100.0, color="black", linewidth=0.8, linestyle="--")
+    ax.set_ylim(0, 110)
+    ax.set_ylabel(f"% of fp32 matrix peak ({peak_tflops:g} TFLOP/s)")
+    ax.set_title("GEMM FP32 on MI355X (Roller-selected HIP MFMA kernels)")
+    for bar, tf, sp in zip(bars, df["Roller TFLOPS"], df["Speedup vs Host"]):
+        text = f"{tf:.0f}" + (f"\n{sp:.0f}x host" if sp else "")
+        ax.text(bar.get_x() + bar.get_width() / 2, bar.get_height() + 1, text, ha="center", va="bottom", fontsize=7)
+    fig.tight_layout()
+    out = Path(path)
+    fig.savefig(out, dpi=150)
+    plt.close(fig)
+    return out
+
+
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(description="Roller fp32 GEMM sweep on MI355X")
     ap.add_argument("--shapes", default="readme", choices=["readme", "full"],
@@ -139,13 +166,16 @@ def main(argv=None) -> None:
     ap.add_argument("--no-baseline", action="store_true")
     ap.add_argument("--csv", default="benchmark_results.csv")
     ap.add_argument("--dump", default=None, help="directory for kernel source / ISA dumps")
+    ap.add_argument("--plot", default=None, help="write a bar chart of the sweep to this image file")
     args = ap.parse_args(argv)
     if args.shapes == "full":
         dims = [2048, 4096, 8192]
         shapes = list(itertools.product(dims, dims, dims))
     else:
         shapes = README_SHAPES
-    benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump)
+    df = benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump)
+    if args.plot:
+        print(f"Chart saved to {plot_results(df, args.plot)}")
 
 
 if __name__ == "__main__":

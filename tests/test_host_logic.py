@@ -140,3 +140,10 @@ def test_readme_shapes_are_the_fourteen():
     assert len(bm.README_SHAPES) == 14 and bm.README_SHAPES[0] == (2048, 2048, 2048)
     assert bm.README_SHAPES[10] == (4096, 8192, 4096) and bm.README_SHAPES[13] == (8192, 4096, 4096)
     assert all(d in (2048, 4096, 8192) for s in bm.README_SHAPES for d in s)
+
+
+def test_plot_results_writes_an_image(tmp_path):
+    import pandas as pd
+    df = pd.DataFrame({"Roller TFLOPS": [139.0, 148.5, 120.0], "Speedup vs Host": [37.0, 40.2, 0]})
+    out = bm.plot_results(df, tmp_path / "sweep.png")
+    assert out.exists() and out.stat().st_size > 5000 and out.read_bytes()[:4] == b"\x89PNG"
