@@ -34,6 +34,24 @@ def test_every_declaration_cites_the_reference_or_says_why_not():
     assert HEADER.count("src/roller.py:") >= 10 and "src/arch.py:" in HEADER and "benchmark.py:" in HEADER
 
 
+def test_config_struct_agrees_in_header_binding_and_integration_stub():
+    # rl_gemm_config is passed by pointer: a binding with fewer fields makes the library read past it
+    struct = re.search(r"typedef struct rl_gemm_config\s*\{(.*?)\}\s*rl_gemm_config;", HEADER, flags=re.S).group(1)
+    struct = re.sub(r"/\*.*?\*/", "", struct, flags=re.S)
+    in_header = [name for decl in re.findall(r"\bint\s+([a-z_,\s]+);", struct) for name in re.findall(r"[a-z_]+", decl)]
+    in_binding = [name for name, _ in hip._GemmConfigC._fields_]
+    in_dataclass = [f.name for f in __import__("dataclasses").fields(GemmConfig)]
+    assert in_header == in_binding == in_dataclass and in_header[-1] == "direct"
+    doc = (ROOT / "INTEGRATION.md").read_text()
+    stub = re.search(r"for n in \((.*?)\)\]", doc, flags=re.S).group(1)
+    assert re.findall(r'"([a-z_]+)"', stub) == in_header
+    # the literal configs of the document are accepted by the library's own validation
+    py_literal = re.search(r"cfg\s*=\s*GemmConfig\(([^)]*)\)", doc).group(1)
+    hip.config_check(GemmConfig(*[int(v) for v in py_literal.split(",")]))
+    c_literal = re.search(r"rl_gemm_config cfg = \{(.*?)\};", doc, flags=re.S).group(1)
+    hip.config_check(GemmConfig(**{k: int(v) for k, v in re.findall(r"\.([a-z_]+)=(\d+)", c_literal)}))
+
+
 def test_template_source_is_embedded_verbatim(hip_lib):
     on_disk = (ROOT / "mlir-roller_amd" / "csrc" / "gemm_f32_mfma.hip").read_text()
     assert hip.template_source() == on_disk
