@@ -139,12 +139,15 @@ const char* rl_gemm_template_source(void);
 int rl_gemm_config_check(const rl_gemm_config* cfg, int* lds_bytes, int* threads);
 
 /* Directory of the on-disk code-object cache (NULL or "" disables it).  Files are keyed by a hash
- * of template source, options and hiprtc version.  The reference has no cache: it rebuilds every
- * (shape, hint) from scratch (src/roller.py:358-387). */
+ * of template source, options and hiprtc version; each file is the code object plus a 16-byte
+ * trailer with its checksum, and a file that fails the check, or that the driver refuses to load,
+ * is recompiled in place.  The reference has no cache: it rebuilds every (shape, hint) from
+ * scratch (src/roller.py:358-387). */
 int rl_set_cache_dir(const char* path);
 
 /* Compiles cfg without touching a device and stores the code object in the cache directory
- * (ahead-of-time warm-up; works on a machine that has no GPU).  *code_size may be NULL. */
+ * (ahead-of-time warm-up; works on a machine that has no GPU).  *code_size (may be NULL) receives
+ * the size of the code object, 16 bytes less than the cache file. */
 int rl_gemm_precompile(const rl_gemm_config* cfg, size_t* code_size);
 
 /* JIT-compiles (or fetches from the in-process / on-disk cache) and loads the kernel for cfg.
@@ -157,7 +160,9 @@ int rl_gemm_plan_threads(const rl_gemm_plan* plan);
 /* Kernel resource usage read from the code object's metadata (-1 if unknown). */
 int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int* sgprs,
                            int* spilled, int* scratch_bytes);
-/* Drops every plan and unloads its module. */
+/* Drops every plan and unloads its module.  Handles obtained earlier stay safe to pass in: the
+ * plan entry points refuse them with RL_ERR_INVALID_ARG.  No counterpart in the reference, which
+ * keeps every CuPy module alive until the process ends. */
 int rl_gemm_plans_clear(void);
 
 /* Enqueues C = A*B (or C += A*B when cfg.accum) for row-major fp32 device matrices

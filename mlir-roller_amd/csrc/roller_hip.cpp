@@ -14,6 +14,7 @@
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <atomic>
 #include <chrono>
 #include <cstdarg>
 #include <cstdio>
@@ -62,9 +63,9 @@ int hip_fail(hipError_t e, const char* what) {
     if (e_ != hipSuccess) return hip_fail(e_, #expr); \
   } while (0)
 
-std::mutex g_mutex;  // guards everything below
-bool g_ready = false;
-int g_device = -1;
+std::mutex g_mutex;  // guards the cache directory, the plan table and initialisation
+std::atomic<bool> g_ready{false};  // read without the lock on every entry point
+std::atomic<int> g_device{-1};
 std::string g_cache_dir;
 
 struct Plan {
@@ -83,6 +84,10 @@ struct rl_gemm_plan : Plan {};
 namespace {
 
 std::map<std::string, rl_gemm_plan*> g_plans;
+// Plans released by rl_gemm_plans_clear: module unloaded, func == nullptr.  The few dozen bytes
+// stay allocated so that a handle a caller still holds is refused instead of dereferencing
+// freed memory.
+std::vector<rl_gemm_plan*> g_released_plans;
 
 uint64_t fnv1a(const void* data, size_t n, uint64_t h) {
   const unsigned char* p = (const unsigned char*)data;
@@ -226,20 +231,54 @@ bool write_file(const std::string& path, const std::vector<char>& data) {
   return ok;
 }
 
-// Code object for cfg: from the disk cache if present, otherwise compiled (and then cached).
-int code_for(const rl_gemm_config& c, std::vector<char>* code, float* compile_ms) {
+// A cache entry is the code object followed by a 16-byte trailer: "RLHC", a format number, and
+// the FNV-1a hash of the code object.  An entry that fails this check (cut short, overwritten,
+// written by another format) is treated as absent.
+constexpr uint32_t kCacheFormat = 1;
+
+void append_trailer(std::vector<char>* data) {
+  const uint64_t h = fnv1a(data->data(), data->size(), 14695981039346656037ull);
+  char t[16] = {'R', 'L', 'H', 'C'};
+  memcpy(t + 4, &kCacheFormat, 4);
+  memcpy(t + 8, &h, 8);
+  data->insert(data->end(), t, t + 16);
+}
+
+bool strip_trailer(std::vector<char>* data) {
+  if (data->size() <= 16 + 64) return false;
+  const char* t = data->data() + data->size() - 16;
+  uint32_t fmt;
+  uint64_t h;
+  memcpy(&fmt, t + 4, 4);
+  memcpy(&h, t + 8, 8);
+  if (memcmp(t, "RLHC", 4) != 0 || fmt != kCacheFormat) return false;
+  data->resize(data->size() - 16);
+  return h == fnv1a(data->data(), data->size(), 14695981039346656037ull) && memcmp(data->data(), "\177ELF", 4) == 0;
+}
+
+// Code object for cfg: from the disk cache if present (unless use_cache is false), otherwise
+// compiled (and then cached).  *from_cache tells the caller which of the two it got.
+int code_for(const rl_gemm_config& c, std::vector<char>* code, float* compile_ms, bool use_cache = true,
+             bool* from_cache = nullptr) {
   if (compile_ms) *compile_ms = 0.0f;
+  if (from_cache) *from_cache = false;
   const std::string path = cache_path(c);
-  if (!path.empty() && read_file(path, code)) return RL_OK;
+  if (use_cache && !path.empty() && read_file(path, code) && strip_trailer(code)) {
+    if (from_cache) *from_cache = true;
+    return RL_OK;
+  }
+  code->clear();
   std::string log;
   const auto t0 = std::chrono::steady_clock::now();
   int rc = compile(rl_gemm_template_begin, "gemm_f32_mfma.hip", config_options(c), code, &log);
   if (rc != RL_OK) return rc;
   if (compile_ms)
     *compile_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
-  if (!path.empty() && !write_file(path, *code)) {
+  if (!path.empty()) {
+    std::vector<char> entry(*code);
+    append_trailer(&entry);
     // A read-only cache directory is not an error for the caller: the kernel is in memory.
-    g_error = "code-object cache not writable: " + path;
+    if (!write_file(path, entry)) g_error = "code-object cache not writable: " + path;
   }
   return RL_OK;
 }
@@ -288,6 +327,8 @@ extern "C" {
 int rl_init(int device) {
   std::lock_guard<std::mutex> lock(g_mutex);
   if (g_ready && g_device == device) return RL_OK;
+  if (g_ready)  // loaded modules, streams and allocations belong to the first device
+    return fail(RL_ERR_INVALID_ARG, "already initialised on device %d; one device per process", g_device.load());
   int count = 0;
   hipError_t e = hipGetDeviceCount(&count);
   if (e != hipSuccess || count <= 0)
@@ -522,7 +563,8 @@ int rl_gemm_precompile(const rl_gemm_config* cfg, size_t* code_size) {
   rc = code_for(*cfg, &code, nullptr);
   if (rc) return rc;
   std::vector<char> check;
-  if (!read_file(cache_path(*cfg), &check)) return fail(RL_ERR_IO, "could not store %s", cache_path(*cfg).c_str());
+  if (!read_file(cache_path(*cfg), &check) || !strip_trailer(&check))
+    return fail(RL_ERR_IO, "could not store %s", cache_path(*cfg).c_str());
   if (code_size) *code_size = code.size();
   return RL_OK;
 }
@@ -545,15 +587,31 @@ int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* co
     return RL_OK;
   }
   std::vector<char> code;
-  rc = code_for(*cfg, &code, compile_ms);
+  bool from_cache = false;
+  rc = code_for(*cfg, &code, compile_ms, true, &from_cache);
   if (rc) return rc;
 
   rl_gemm_plan* p = new rl_gemm_plan();
   p->cfg = *cfg;
   p->lds_bytes = lds;
   p->threads = threads;
-  hipError_t e = hipModuleLoadData(&p->module, code.data());
-  if (e == hipSuccess) e = hipModuleGetFunction(&p->func, p->module, "gemm_kernel");
+  hipError_t e = hipSuccess;
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    e = hipModuleLoadData(&p->module, code.data());
+    if (e == hipSuccess) e = hipModuleGetFunction(&p->func, p->module, "gemm_kernel");
+    if (e == hipSuccess || !from_cache) break;
+    // A cached file that does not load (damaged, or written for another driver) is replaced once.
+    (void)hipGetLastError();
+    if (p->module) (void)hipModuleUnload(p->module);
+    p->module = nullptr;
+    p->func = nullptr;
+    from_cache = false;
+    rc = code_for(*cfg, &code, compile_ms, false, nullptr);
+    if (rc) {
+      delete p;
+      return rc;
+    }
+  }
   if (e == hipSuccess && lds > 64 * 1024 && opt_in_lds(p->func, lds) != RL_OK) e = hipErrorInvalidValue;
   if (e != hipSuccess) {
     if (p->module) (void)hipModuleUnload(p->module);
@@ -573,6 +631,7 @@ int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* co
 
 int rl_gemm_plan_function(const rl_gemm_plan* plan, rl_function* out) {
   if (!plan || !out) return fail(RL_ERR_INVALID_ARG, "rl_gemm_plan_function: NULL argument");
+  if (!plan->func) return fail(RL_ERR_INVALID_ARG, "plan was released by rl_gemm_plans_clear");
   *out = plan->func;
   return RL_OK;
 }
@@ -599,7 +658,9 @@ int rl_gemm_plans_clear(void) {
       hipError_t e = hipModuleUnload(kv.second->module);
       if (e != hipSuccess) rc = hip_fail(e, "hipModuleUnload");
     }
-    delete kv.second;
+    kv.second->module = nullptr;
+    kv.second->func = nullptr;
+    g_released_plans.push_back(kv.second);
   }
   g_plans.clear();
   return rc;
@@ -608,6 +669,7 @@ int rl_gemm_plans_clear(void) {
 int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
                         int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream) {
   if (!plan) return fail(RL_ERR_INVALID_ARG, "plan is NULL");
+  if (!plan->func) return fail(RL_ERR_INVALID_ARG, "plan was released by rl_gemm_plans_clear");
   const rl_gemm_config& c = plan->cfg;
   if (M < 0 || N < 0 || K < 0) return fail(RL_ERR_INVALID_ARG, "negative dimension (M=%d N=%d K=%d)", M, N, K);
   if (M == 0 || N == 0) return RL_OK;

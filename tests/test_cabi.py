@@ -113,9 +113,13 @@ def test_precompile_fills_the_disk_cache(hip_lib, tmp_path):
         cfg = GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 1)
         size = hip.precompile(cfg)
         files = list(tmp_path.glob("gemm_*.hsaco"))
-        assert len(files) == 1 and files[0].stat().st_size == size
+        assert len(files) == 1 and files[0].stat().st_size == size + 16               # code object + checksum trailer
         stamp = files[0].stat().st_mtime_ns
         assert hip.precompile(cfg) == size and files[0].stat().st_mtime_ns == stamp   # cache hit: not rewritten
+        good = files[0].read_bytes()
+        for damaged in (b"not a code object", good[:-1], good[:100] + bytes([good[100] ^ 1]) + good[101:]):
+            files[0].write_bytes(damaged)                                                # fails the checksum: replaced
+            assert hip.precompile(cfg) == size and files[0].read_bytes() == good
         hip.precompile(GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 0))
         assert len(list(tmp_path.glob("gemm_*.hsaco"))) == 2                             # key covers every field
         hip.set_cache_dir(None)

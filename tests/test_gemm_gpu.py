@@ -230,6 +230,33 @@ def test_plan_cache_and_one_shot_entry_point(device):
     assert np.array_equal(dC.get(), go.c_gemm_f32(A, B))
 
 
+def test_released_plans_and_damaged_cache_entries(device, tmp_path):
+    """rl_gemm_plans_clear leaves old handles refusable (not dangling); a cache file that fails
+    its checksum is recompiled in place instead of being handed to the loader."""
+    cfg = GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4, 1)
+    A, B = go.make_inputs(70, 92, 52, seed=5, distribution="integer")
+    want = go.gemm_f32(A, B)
+    old_dir = hip.DEFAULT_CACHE_DIR
+    try:
+        hip.set_cache_dir(tmp_path)
+        hip.lib().rl_gemm_plans_clear()
+        stale = GemmPlan(cfg)
+        assert np.array_equal(run_gemm(cfg, A, B), want)
+        hip.lib().rl_gemm_plans_clear()
+        dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray((70, 92))
+        with pytest.raises(HipError) as err:
+            stale.launch(dA, dB, dC, 70, 92, 52)
+        assert "released" in str(err.value)
+        (entry,) = tmp_path.glob("gemm_*.hsaco")
+        good = entry.read_bytes()
+        entry.write_bytes(good[:64] + b"\0" * (len(good) - 64))
+        assert np.array_equal(run_gemm(cfg, A, B), want)            # reloaded through a fresh compile
+        assert entry.read_bytes() == good
+    finally:
+        hip.lib().rl_gemm_plans_clear()
+        hip.set_cache_dir(old_dir)
+
+
 def test_low_level_module_api_like_the_reference_uses_cupy(device):
     src = r'''extern "C" __global__ void axpy(float a, const float* x, float* y, int n) {
         int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -299,6 +326,45 @@ def test_m0_to_m13_exact_on_integer_inputs_at_full_size(device):
         func(func.grid_dims(), func.block_dims(), (dA, dB, dC))
         hip.synchronize()
         assert np.array_equal(dC.get(), go.gemm_f32(A, B)), shape
+
+
+def small_integer_matrix(rows, cols, seed):
+    """Integer-valued float32 matrix in {-2..2} built from two short random vectors (cheap at
+    billions of elements, and not constant along any row, column or diagonal)."""
+    rng = np.random.default_rng(seed)
+    r = rng.integers(0, 5, size=(rows, 1), dtype=np.int8)
+    c = rng.integers(0, 5, size=(1, cols), dtype=np.int8)
+    return ((r + c) % 5 - 2).astype(np.float32)
+
+
+# One operand beyond 4 GiB each: tile base addresses need 64-bit arithmetic and the byte ranges of
+# the buffer resources exceed what their 32-bit size field holds.  (M, N, K), config.
+BEYOND_4GIB = [
+    ("A", (65792, 256, 16384), GemmConfig(256, 256, 32, 128, 128, 32, 3, 0, 0, 4, 0, 3, 8, 0, 1)),
+    ("B", (256, 65792, 16384), GemmConfig(256, 256, 32, 128, 128, 32, 3, 0, 0, 4, 0, 3, 8, 0, 1)),
+    ("C", (32768, 32900, 32), GemmConfig(256, 256, 32, 64, 128, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1)),
+    ("C-staged", (32768, 32900, 40), GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1)),
+]
+
+
+@pytest.mark.parametrize("which,shape,cfg", BEYOND_4GIB, ids=[b[0] for b in BEYOND_4GIB])
+def test_operands_larger_than_4_gib(device, which, shape, cfg):
+    """Maximum sizes: with entries in {-2..2} and K <= 16384 every partial sum is an integer
+    below 2^24, so the float32 host GEMM is exact in any order and the comparison is bit-for-bit."""
+    M, N, K = shape
+    say("beyond 4 GiB:", which, shape, cfg.tag())
+    assert max(M * K, K * N, M * N) * 4 > 1 << 32
+    A, B = small_integer_matrix(M, K, 1), small_integer_matrix(K, N, 2)
+    want = A @ B
+    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B)
+    dC = DeviceArray((M, N))
+    dC.fill_bytes(0xFF)
+    GemmPlan(cfg).launch(dA, dB, dC, M, N, K)
+    hip.synchronize()
+    got = dC.get()
+    del dA, dB, dC
+    for r0 in range(0, M, 4096):                       # in slabs: no 4 GiB boolean temporaries
+        assert np.array_equal(got[r0:r0 + 4096], want[r0:r0 + 4096]), (which, r0)
 
 
 def test_handle_checks_grid_and_block(device):
