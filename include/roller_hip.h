@@ -71,6 +71,9 @@ typedef struct rl_gemm_config {
   int accum;       /* 0: C = A*B, 1: C += A*B (linalg.matmul semantics, roller.py:62)*/
   int direct;      /* 1: global loads write LDS directly (no staging registers, swizzled
                       A rows); needs stages=3, vec=4, pad_a=pad_b=0, bk a power of 2 */
+  int trans_b;     /* 1: the second operand is Bt[N][ldb>=K], C = A*Bt^T (the [spatial, reduce]
+                      layout of MatmulConfig.get_input_shapes, src/analyze.py:33-41); pad_b then
+                      pads the K-contiguous rows of its LDS tile like pad_a                   */
 } rl_gemm_config;
 
 /* ---- library / device ---------------------------------------------------------------------- */
@@ -133,7 +136,8 @@ int rl_sync(void);
 const char* rl_gemm_template_source(void);
 
 /* Checks cfg against the template's constraints without compiling.  *lds_bytes (may be NULL)
- * receives the dynamic LDS size = min(stages,2) * (bm*(bk+pad_a) + bk*(bn+pad_b)) * 4, the padded
+ * receives the dynamic LDS size = min(stages,2) * (bm*(bk+pad_a) + bk*(bn+pad_b)) * 4
+ * (bn*(bk+pad_b) for the second term when trans_b), the padded
  * counterpart of hint.smem_cost * pipeline_depth (src/roller.py:385); *threads (may be NULL)
  * receives 64 * (bm/wm) * (bn/wn). */
 int rl_gemm_config_check(const rl_gemm_config* cfg, int* lds_bytes, int* threads);
@@ -166,7 +170,7 @@ int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int
 int rl_gemm_plans_clear(void);
 
 /* Enqueues C = A*B (or C += A*B when cfg.accum) for row-major fp32 device matrices
- * A[M,lda>=K], B[K,ldb>=N], C[M,ldc>=N].  Grid is (ceil(N/bn), ceil(M/bm)) as at
+ * A[M,lda>=K], B[K,ldb>=N] (Bt[N,ldb>=K] when cfg.trans_b), C[M,ldc>=N].  Grid is (ceil(N/bn), ceil(M/bm)) as at
  * src/roller.py:536 (the reference floors; ragged tiles are predicated here when cfg.edge).
  * Rejects, with RL_ERR_INVALID_ARG and before anything is launched, shapes the plan was not built
  * for: vec=4 with K, N or a leading dimension not a multiple of 4 or a base pointer not 16-byte

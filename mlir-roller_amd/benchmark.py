@@ -115,6 +115,8 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
             "Hints Failed": failed,
             "Search (s)": search_s,
             "Compile (s)": compile_s,
+            "Min Launch (ms)": best_info.get("min_ms", float("nan")),
+            "Median Launch (ms)": best_info.get("median_ms", float("nan")),
             "Normwise Error": best_info.get("normwise", float("nan")),
             "Max Abs Error": best_info.get("max_abs", float("nan")),
             "Max Abs Bound": best_info.get("bound", float("nan")),

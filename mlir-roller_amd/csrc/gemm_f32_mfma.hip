@@ -1,4 +1,5 @@
 // fp32 GEMM kernel template for gfx950 (MI355X, CDNA4):  C[M,N] = A[M,K] * B[K,N]
+// (or, with TRANS_B, C[M,N] = A[M,K] * Bt[N,K]^T)
 //
 // Row-major operands, fp32 MFMA with fp32 accumulators.  The file is a template in the
 // preprocessor sense: every rTile parameter arrives as a -D define from the JIT (hiprtc) or from
@@ -38,6 +39,12 @@
 //               instead the 16-byte chunks of every A row are XOR-swizzled with the row number
 //               (on the load side by choosing which global chunk a lane fetches, on the read
 //               side in the fragment address), which keeps the 128-bit A reads conflict-free.
+//   TRANS_B     1 = the second operand is given transposed, Bt[N][ldb >= K] (K contiguous, the
+//               layout in which the policy models both inputs, /root/reference/src/analyze.py:33-41).
+//               Its tile then sits in LDS like the A tile ([BN][BK+PAD_B], swizzled under DIRECT)
+//               and a lane reads four consecutive k of one column with one ds_read_b128.  LDS row
+//               r of the tile holds the column that block r/MI hands to lane r%MI (see below), so
+//               consecutive lanes read consecutive rows and C leaves in the same vector stores.
 //
 // Layout trick that removes every LDS bank conflict and every register shuffle on the read side:
 // an MFMA sums over its k slots, and a GEMM does not care which MFMA block owns which column, so
@@ -111,6 +118,9 @@
 #ifndef DIRECT
 #define DIRECT 0
 #endif
+#ifndef TRANS_B
+#define TRANS_B 0
+#endif
 
 #define NWM (BM / WM)
 #define NWN (BN / WN)
@@ -123,9 +133,14 @@
 #define VN (TN >= 4 ? 4 : TN)
 #define NVB (TN / VN)
 #define LDA_S (BK + PAD_A)
+#if TRANS_B
+#define LDB_S (BK + PAD_B)
+#define B_STAGE (BN * LDB_S)
+#else
 #define LDB_S (BN + PAD_B)
-#define A_STAGE (BM * LDA_S)
 #define B_STAGE (BK * LDB_S)
+#endif
+#define A_STAGE (BM * LDA_S)
 #define STAGE_FLOATS (A_STAGE + B_STAGE)
 #define LDS_BUFS (STAGES >= 2 ? 2 : 1)
 #define SUPERS (BK / KSUPER) /* MFMA groups per K step, each fed by one round of fragment reads */
@@ -149,6 +164,7 @@ static_assert(WM % MI == 0 && WN % MI == 0, "MFMA block must divide wave tile");
 static_assert(TN == 1 || TN == 2 || TN % 4 == 0, "column blocks per wave: 1, 2 or a multiple of 4");
 static_assert(BK % KSUPER == 0, "BK must be a multiple of 4*(64/MI)");
 static_assert(PAD_A % 4 == 0 && PAD_B % 4 == 0, "LDS rows stay 16-byte aligned");
+static_assert(TRANS_B == 0 || TRANS_B == 1, "TRANS_B is a flag");
 static_assert(NT <= 1024, "at most 16 waves per workgroup");
 static_assert(STAGES >= 1 && STAGES <= 3, "pipeline depth 1, 2 or 3");
 static_assert(VEC == 4 || VEC == 1, "global access width");
@@ -236,6 +252,15 @@ DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool
 #endif
 }
 
+#if TRANS_B
+// Column of the block tile that LDS row `row` of the Bt tile holds.  Block bj of a wave owns the
+// columns (bj/VN)*MI*VN + VN*lane + bj%VN of its wave tile; row bj*MI + lane holds that column.
+DEV int bt_col_of_row(int row) {
+  const int w = row / WN, q = row % WN, v = q / (MI * VN), rem = q % (MI * VN);
+  return w * WN + v * MI * VN + VN * (rem % MI) + rem / MI;
+}
+#endif
+
 // Maps the hardware workgroup id to a tile of C.
 DEV bool tile_of_workgroup(int nbm, int nbn, int& tile_m, int& tile_n) {
   int pid = blockIdx.y * gridDim.x + blockIdx.x;
@@ -307,19 +332,42 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
   for (int i = 0; i < B_PER_T; ++i) {
     const int u = tid + i * NT;
+    const bool in = (B_UNITS % NT == 0 || u < B_UNITS);
+#if TRANS_B
+    // as for A, with the row of the tile standing for a (permuted) column of C; b_krow holds the
+    // k offset of the unit inside the K step
+#if DIRECT
+    const int row = u / CPR, c = (u % CPR) ^ ((row / RPL) % SWZ_N);
+#else
+    const int row = u / (BK / 4), c = u % (BK / 4);
+#endif
+    const int col = bt_col_of_row(row);
+    b_goff[i] = (unsigned)(col * ldb + c * 4) * 4u;
+    b_soff[i] = row * LDB_S + c * 4;
+    b_krow[i] = c * 4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) b_ok[i][e] = in && (!EDGE || n0 + col < N);
+#else
     const int krow = u / (BN / 4), c = u % (BN / 4);
     b_goff[i] = (unsigned)(krow * ldb + c * 4) * 4u;
     b_soff[i] = krow * LDB_S + c * 4;
     b_krow[i] = krow;
-    const bool in = (B_UNITS % NT == 0 || u < B_UNITS);
 #pragma unroll
     for (int e = 0; e < 4; ++e) b_ok[i][e] = in && (!EDGE || n0 + c * 4 + e < N);
+#endif
   }
 
   const float* Ag = A + (long)m0 * lda;
-  const float* Bg = B + n0;
   long a_rem = ((long)(M - m0 - 1) * lda + K) * 4;        // valid bytes from Ag to the end of A
+#if TRANS_B
+  const float* Bg = B + (long)n0 * ldb;
+  long b_rem = ((long)(N - n0 - 1) * ldb + K) * 4;        // valid bytes from Bg to the end of Bt
+#define B_STEP(k0) (long)(k0)                             /* floats from Bg to K step k0 */
+#else
+  const float* Bg = B + n0;
   long b_rem = ((long)(K - 1) * ldb + (N - n0)) * 4;      // valid bytes from Bg to the end of B
+#define B_STEP(k0) ((long)(k0) * ldb)
+#endif
 
 #if !DIRECT
   v4f ra[A_PER_T], rb[B_PER_T];
@@ -335,7 +383,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const int k0 = kt * BK;
     const bool live = kt < KT;
     const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, live ? a_rem - (long)k0 * 4 : 0);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + (long)k0 * ldb, live ? b_rem - (long)k0 * ldb * 4 : 0);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + B_STEP(k0), live ? b_rem - B_STEP(k0) * 4 : 0);
     float* As = lds + stage * STAGE_FLOATS;
     float* Bs = As + A_STAGE;
 #pragma unroll
@@ -350,7 +398,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < B_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (B_UNITS % NT == 0 || first < B_UNITS) {
-        const bool ok = b_ok[i][0] && (!EDGE || k0 + b_krow[i] < K);
+        const bool ok = b_ok[i][0] && (!EDGE || k0 + b_krow[i] < K);  // K % 4 == 0: a chunk is in or out as a whole
         __builtin_amdgcn_raw_ptr_buffer_load_lds(br, (lds_ptr_t)(Bs + first * 4), 16, ok ? b_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -364,7 +412,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const int k0 = kt * BK;
     const bool live = kt < KT;
     const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, live ? a_rem - (long)k0 * 4 : 0);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + (long)k0 * ldb, live ? b_rem - (long)k0 * ldb * 4 : 0);
+    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + B_STEP(k0), live ? b_rem - B_STEP(k0) * 4 : 0);
 #pragma unroll
     for (int i = 0; i < A_PER_T; ++i) {
       const int k = k0 + a_kcol[i];
@@ -374,9 +422,16 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     }
 #pragma unroll
     for (int i = 0; i < B_PER_T; ++i) {
+#if TRANS_B
+      const int k = k0 + b_krow[i];
+      rb[i] = load_unit(br, b_goff[i],
+                        b_ok[i][0] && (!EDGE || k + 0 < K), b_ok[i][1] && (!EDGE || k + 1 < K),
+                        b_ok[i][2] && (!EDGE || k + 2 < K), b_ok[i][3] && (!EDGE || k + 3 < K));
+#else
       const bool kin = !EDGE || k0 + b_krow[i] < K;
       rb[i] = load_unit(br, b_goff[i], b_ok[i][0] && kin, b_ok[i][1] && kin, b_ok[i][2] && kin,
                         b_ok[i][3] && kin);
+#endif
     }
   };
 
@@ -408,13 +463,24 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #else
   const int a_frag = (wm0 + lr) * LDA_S + 4 * lg;   // + bi*MI*LDA_S + kk
 #endif
+#if TRANS_B && DIRECT
+  const int b_frag = (wn0 + lr) * LDB_S;                // + bj*MI*LDB_S + swizzled chunk of the round
+#elif TRANS_B
+  const int b_frag = (wn0 + lr) * LDB_S + 4 * lg;       // + bj*MI*LDB_S + kk
+#else
   const int b_frag = (4 * lg) * LDB_S + wn0 + VN * lr;  // + (kk+t)*LDB_S + v*MI*VN
+#endif
 
   // One round of LDS fragment reads: TM 128-bit reads of A (four consecutive k each) and, for each
-  // of the four k slots, NVB vector reads of B.  Feeds 4*TM*TN MFMAs.
+  // of the four k slots, NVB vector reads of B (TRANS_B: TN 128-bit reads, four consecutive k of
+  // one column each).  Feeds 4*TM*TN MFMAs.
   struct frag_t {
     v4f a[TM];
+#if TRANS_B
+    v4f b[TN];
+#else
     bvec_t b[4][NVB];
+#endif
   };
   auto read_frags = [&](frag_t& f, int stage, int kk) {
     const float* As = lds + stage * STAGE_FLOATS;
@@ -425,10 +491,18 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #else
     for (int bi = 0; bi < TM; ++bi) f.a[bi] = *(const v4f*)&As[a_frag + bi * MI * LDA_S + kk];
 #endif
+#if TRANS_B && DIRECT
+#pragma unroll
+    for (int bj = 0; bj < TN; ++bj) f.b[bj] = *(const v4f*)&Bs[b_frag + bj * MI * LDB_S + a_round[kk / KSUPER]];
+#elif TRANS_B
+#pragma unroll
+    for (int bj = 0; bj < TN; ++bj) f.b[bj] = *(const v4f*)&Bs[b_frag + bj * MI * LDB_S + kk];
+#else
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int v = 0; v < NVB; ++v) f.b[t][v] = *(const bvec_t*)&Bs[b_frag + (kk + t) * LDB_S + v * MI * VN];
+#endif
   };
   auto mfma_frags = [&](const frag_t& f, int t0 = 0, int t1 = 4) {
 #pragma unroll
@@ -437,7 +511,9 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       for (int bi = 0; bi < TM; ++bi)
 #pragma unroll
         for (int bj = 0; bj < TN; ++bj) {
-#if VN == 1
+#if TRANS_B
+          const float bval = f.b[bj][t];
+#elif VN == 1
           const float bval = f.b[t][bj];
 #else
           const float bval = f.b[t][bj / VN][bj % VN];
@@ -471,7 +547,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // P = which of the two fragment sets holds round 0 of this step (compile-time, so that the
     // sets stay in fixed registers); the set alternates every round.
     // MFMAs and fragment reads per round; LDS writes and global loads per K step
-    constexpr int G = 4 * TM * TN, R = TM + 4 * NVB, W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
+    constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NVB), W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
 
     auto step = [&](auto parity, int kt) {
       constexpr int P = decltype(parity)::value;

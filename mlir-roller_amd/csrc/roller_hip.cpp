@@ -129,9 +129,10 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
     if ((c.bm * c.bk / 4) % 64 || (c.bk * c.bn / 4) % 64)
       return fail(RL_ERR_INVALID_ARG, "direct=1 needs bm*bk and bk*bn to be multiples of 256 (whole waves of 16-byte units)");
   }
+  if ((c.trans_b | 1) != 1) return fail(RL_ERR_INVALID_ARG, "trans_b is 0 or 1");
   const int nt = 64 * (c.bm / c.wm) * (c.bn / c.wn);
   if (nt > 1024) return fail(RL_ERR_INVALID_ARG, "%d threads per workgroup exceed 1024", nt);
-  const long lds = (long)(c.stages >= 2 ? 2 : 1) * ((long)c.bm * (c.bk + c.pad_a) + (long)c.bk * (c.bn + c.pad_b)) * 4;
+  const long lds = (long)(c.stages >= 2 ? 2 : 1) * ((long)c.bm * (c.bk + c.pad_a) + (c.trans_b ? (long)c.bn * (c.bk + c.pad_b) : (long)c.bk * (c.bn + c.pad_b))) * 4;
   if (lds > 160 * 1024) return fail(RL_ERR_INVALID_ARG, "%ld bytes of LDS exceed the 160 KB of a CU", lds);
   if (lds_bytes) *lds_bytes = (int)lds;
   if (threads) *threads = nt;
@@ -145,6 +146,7 @@ std::vector<std::string> config_options(const rl_gemm_config& c) {
   def("STAGES", c.stages); def("PAD_A", c.pad_a); def("PAD_B", c.pad_b); def("VEC", c.vec);
   def("EDGE", c.edge); def("SWZ", c.swz); def("GROUP", c.group > 0 ? c.group : 1); def("ACCUM", c.accum);
   def("DIRECT", c.direct);
+  def("TRANS_B", c.trans_b);
   return o;
 }
 
@@ -674,8 +676,8 @@ int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B
   if (M < 0 || N < 0 || K < 0) return fail(RL_ERR_INVALID_ARG, "negative dimension (M=%d N=%d K=%d)", M, N, K);
   if (M == 0 || N == 0) return RL_OK;
   if (!C || (K > 0 && (!A || !B))) return fail(RL_ERR_INVALID_ARG, "NULL matrix pointer");
-  if (lda < K || ldb < N || ldc < N)
-    return fail(RL_ERR_INVALID_ARG, "leading dimension too small (lda=%d K=%d, ldb=%d ldc=%d N=%d)", lda, K, ldb, ldc, N);
+  if (lda < K || ldb < (c.trans_b ? K : N) || ldc < N)
+    return fail(RL_ERR_INVALID_ARG, "leading dimension too small (lda=%d K=%d, ldb=%d ldc=%d N=%d, trans_b=%d)", lda, K, ldb, ldc, N, c.trans_b);
   if (c.vec == 4) {
     if (K % 4 || N % 4 || lda % 4 || ldb % 4 || ldc % 4)
       return fail(RL_ERR_INVALID_ARG, "vec=4 kernel needs K, N, lda, ldb, ldc to be multiples of 4 (K=%d N=%d lda=%d ldb=%d ldc=%d)", K, N, lda, ldb, ldc);
@@ -688,7 +690,7 @@ int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B
     return fail(RL_ERR_INVALID_ARG, "edge=0 kernel needs bm|M, bn|N, bk|K (tile %dx%dx%d, problem %dx%dx%d)", c.bm, c.bn, c.bk, M, N, K);
   // In-tile byte offsets are 32-bit inside the kernel; 0x80000000 is reserved as "out of range".
   const long lim = 0x7fffffffL;
-  if ((long)c.bm * lda * 4 + (long)c.bk * 4 > lim || (long)c.bk * ldb * 4 + (long)c.bn * 4 > lim ||
+  if ((long)c.bm * lda * 4 + (long)c.bk * 4 > lim || (c.trans_b ? (long)c.bn * ldb * 4 + (long)c.bk * 4 : (long)c.bk * ldb * 4 + (long)c.bn * 4) > lim ||
       (long)c.bm * ldc * 4 + (long)c.bn * 4 > lim)
     return fail(RL_ERR_INVALID_ARG, "leading dimension too large for 32-bit in-tile offsets");
   const long nbm = ((long)M + c.bm - 1) / c.bm, nbn = ((long)N + c.bn - 1) / c.bn;

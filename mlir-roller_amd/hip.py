@@ -61,7 +61,7 @@ class DeviceProps(C.Structure):
 class _GemmConfigC(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "bm", "bn", "bk", "wm", "wn", "mi", "stages", "pad_a", "pad_b", "vec", "edge", "swz",
-        "group", "accum", "direct")]
+        "group", "accum", "direct", "trans_b")]
 
 
 @dataclass(frozen=True)
@@ -83,6 +83,7 @@ class GemmConfig:
     group: int = 8
     accum: int = 0
     direct: int = 0
+    trans_b: int = 0
 
     def to_c(self) -> _GemmConfigC:
         return _GemmConfigC(*(getattr(self, f.name) for f in fields(self)))
@@ -93,12 +94,13 @@ class GemmConfig:
 
     @property
     def lds_bytes(self) -> int:
-        return min(self.stages, 2) * (self.bm * (self.bk + self.pad_a) + self.bk * (self.bn + self.pad_b)) * 4
+        b_tile = self.bn * (self.bk + self.pad_b) if self.trans_b else self.bk * (self.bn + self.pad_b)
+        return min(self.stages, 2) * (self.bm * (self.bk + self.pad_a) + b_tile) * 4
 
     def tag(self) -> str:
         return (f"b{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_mi{self.mi}_s{self.stages}"
                 f"_p{self.pad_a}.{self.pad_b}_v{self.vec}_e{self.edge}_z{self.swz}.{self.group}"
-                f"_a{self.accum}" + ("_d1" if self.direct else ""))
+                f"_a{self.accum}" + ("_d1" if self.direct else "") + ("_tb" if self.trans_b else ""))
 
 
 # --------------------------------------------------------------------------------------------
@@ -455,8 +457,9 @@ class GemmPlan:
     def launch(self, A, B, Cm, M: int, N: int, K: int, lda: Optional[int] = None,
                ldb: Optional[int] = None, ldc: Optional[int] = None, stream=None) -> None:
         ptr = lambda x: x.ptr if isinstance(x, DeviceArray) else int(x)
+        width_b = K if self.cfg.trans_b else N
         check(lib().rl_gemm_plan_launch(self.handle, ptr(A), ptr(B), ptr(Cm), M, N, K,
-                                        K if lda is None else lda, N if ldb is None else ldb,
+                                        K if lda is None else lda, width_b if ldb is None else ldb,
                                         N if ldc is None else ldc, _stream_handle(stream)))
 
 
@@ -466,6 +469,7 @@ def gemm_f32(cfg: GemmConfig, A, B, Cm, M: int, N: int, K: int, lda=None, ldb=No
     init()
     ptr = lambda x: x.ptr if isinstance(x, DeviceArray) else int(x)
     c = cfg.to_c()
+    width_b = K if cfg.trans_b else N
     check(lib().rl_gemm_f32(C.byref(c), ptr(A), ptr(B), ptr(Cm), M, N, K,
-                            K if lda is None else lda, N if ldb is None else ldb,
+                            K if lda is None else lda, width_b if ldb is None else ldb,
                             N if ldc is None else ldc, _stream_handle(stream)))

@@ -36,13 +36,14 @@ WARMUP_MS = 40.0             # load queued ahead of the timed launches of run_ev
 
 
 def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: int = 2,
-                        accumulate: bool = False) -> GemmConfig:
+                        accumulate: bool = False, trans_b: bool = False) -> GemmConfig:
     """Template parameters for one hint.
 
     block_tile -> BM, BN; rstep -> BK; wave_tile -> WM, WN (derived from the thread count when
     the hint comes from a device model without matrix cores); pipeline_depth -> pipeline stages
     (the template has 1 to 3; from 2 on it keeps two LDS buffers).  Ragged problems switch on predication, and problems whose K, N
-    are not multiples of 4 fall back to dword global accesses.
+    are not multiples of 4 fall back to dword global accesses.  ``trans_b`` selects the kernel
+    whose second operand is stored as Bt[N, K].
     """
     bm, bn = hint.block_tile
     bk = hint.rstep
@@ -69,10 +70,14 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
                  and (bm * bk // 4) % 64 == 0 and (bk * bn // 4) % 64 == 0)
     # otherwise (bk + pad)/4 odd keeps the 128-bit reads of LDS-A free of bank conflicts
     pad_a = 0 if direct else (4 if (bk // 4) % 2 == 0 else 0)
+    # a transposed second operand sits in LDS like A and wants the same padding, LDS permitting
+    pad_b = pad_a if trans_b else 0
+    if pad_b and min(stages, 2) * (bm * (bk + pad_a) + bn * (bk + pad_b)) * 4 > MI355X().lds_bytes:
+        pad_b = 0
     return GemmConfig(
-        bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi, stages=stages, pad_a=pad_a, pad_b=0, vec=vec,
+        bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi, stages=stages, pad_a=pad_a, pad_b=pad_b, vec=vec,
         edge=0 if (M % bm == 0 and N % bn == 0 and K % bk == 0) else 1,
-        swz=3, group=8, accum=1 if accumulate else 0, direct=direct,
+        swz=3, group=8, accum=1 if accumulate else 0, direct=direct, trans_b=1 if trans_b else 0,
     )
 
 
@@ -117,7 +122,7 @@ class KernelHandle:
     def __call__(self, grid_dims, block_dims, args, shared_mem: int = 0, stream=None) -> None:
         if len(args) == 3:
             c = self.config
-            dims = (c.M, c.N, c.K, c.K, c.N, c.N)
+            dims = (c.M, c.N, c.K, c.K, c.K if self.gemm_config.trans_b else c.N, c.N)
         elif len(args) == 9:
             dims = tuple(int(v) for v in args[3:])
         else:
@@ -148,15 +153,16 @@ class Compiler:
     """
 
     def __init__(self, config: MatmulConfig, hint: TileDict, pipeline_depth: int = 2,
-                 dump_path: Optional[Path] = None, accumulate: bool = False):
+                 dump_path: Optional[Path] = None, accumulate: bool = False, trans_b: bool = False):
         self.config = config
         self.hint = hint
         self.pipeline_depth = pipeline_depth
         self.dump_path = Path(dump_path) if dump_path else None
         self.accumulate = accumulate
+        self.trans_b = trans_b
 
     def compile(self) -> KernelHandle:
-        gemm_config = hint_to_gemm_config(self.config, self.hint, self.pipeline_depth, self.accumulate)
+        gemm_config = hint_to_gemm_config(self.config, self.hint, self.pipeline_depth, self.accumulate, self.trans_b)
         hip.config_check(gemm_config)
         plan = GemmPlan(gemm_config)
         handle = KernelHandle(plan, self.config, gemm_config, self.hint)
@@ -257,7 +263,8 @@ def run_eval(cuda_func: KernelHandle, pipeline_depth, hint: TileDict, repeat_tim
     """Protocol of the reference's ``run_eval`` (roller.py:525-586): one checked launch, one
     more single launch, warm-ups (ten, or as many as fill ``WARMUP_MS``), then ``repeat_times``
     launches between two events.
-    Returns ``(ms_per_launch, gflops)``; details land in ``cuda_func.last_eval``.
+    Returns ``(ms_per_launch, gflops)``; details (error measures, minimum and median of
+    per-launch event pairs) land in ``cuda_func.last_eval``.
 
     Unlike the reference, which only prints on a mismatch, a result outside the tolerances
     raises, so that a wrong kernel can never be picked as the fastest one.
@@ -266,10 +273,10 @@ def run_eval(cuda_func: KernelHandle, pipeline_depth, hint: TileDict, repeat_tim
     M, N, K = cfg.M, cfg.N, cfg.K
     case = _host_case(cfg, seed, distribution)
     A, B, C32 = case[0], case[1], case[2]
-    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B)
+    g = cuda_func.gemm_config
+    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B.T if g.trans_b else B)
     dC = DeviceArray.zeros((M, N))
 
-    g = cuda_func.gemm_config
     grid_dims = (-(-N // g.bn), -(-M // g.bm))  # the reference floors here; ragged tiles exist now
     block_dims = cuda_func.block_dims()
     shared_memory_usage = max(hint.smem_cost * int(pipeline_depth), cuda_func.shared_mem_bytes)
@@ -294,11 +301,22 @@ def run_eval(cuda_func: KernelHandle, pipeline_depth, hint: TileDict, repeat_tim
         for _ in range(repeat_times):
             cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
     t_gpu = hip.get_elapsed_time(start_gpu, end_gpu)
+    # Per-launch spread: a second batch with an event after every launch (recording an event
+    # does not idle the GPU, so the clock stays up), read back after one final wait.
+    marks = [Event() for _ in range(repeat_times + 1)]
+    marks[0].record()
+    for mark in marks[1:]:
+        cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
+        mark.record()
+    marks[-1].synchronize()
+    each = sorted(hip.get_elapsed_time(a, b) for a, b in zip(marks, marks[1:]))
 
     flops = 2 * M * N * K
     gflops = repeat_times * flops * 1e-9 / (t_gpu / 1000)
     print(f"t={t_gpu / repeat_times:.6f} ms GFLOPS={gflops:.6f}")
     info.update(ms=t_gpu / repeat_times, gflops=gflops)
+    if each:
+        info.update(min_ms=each[0], median_ms=each[len(each) // 2])
     cuda_func.last_eval = info
     return t_gpu / repeat_times, gflops
 

@@ -41,7 +41,7 @@ def test_config_struct_agrees_in_header_binding_and_integration_stub():
     in_header = [name for decl in re.findall(r"\bint\s+([a-z_,\s]+);", struct) for name in re.findall(r"[a-z_]+", decl)]
     in_binding = [name for name, _ in hip._GemmConfigC._fields_]
     in_dataclass = [f.name for f in __import__("dataclasses").fields(GemmConfig)]
-    assert in_header == in_binding == in_dataclass and in_header[-1] == "direct"
+    assert in_header == in_binding == in_dataclass and in_header[-2:] == ["direct", "trans_b"]
     doc = (ROOT / "INTEGRATION.md").read_text()
     stub = re.search(r"for n in \((.*?)\)\]", doc, flags=re.S).group(1)
     assert re.findall(r'"([a-z_]+)"', stub) == in_header

@@ -31,7 +31,8 @@ def say(*a):
 def run_gemm(cfg: GemmConfig, A: np.ndarray, B: np.ndarray, c_init=None) -> np.ndarray:
     M, K = A.shape
     N = B.shape[1]
-    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B)
+    # a trans_b kernel takes the second operand as Bt[N, K]
+    dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B.T if cfg.trans_b else B)
     if c_init is None:
         dC = DeviceArray((M, N))
         dC.fill_bytes(0xFF)  # NaN pattern: every element must be overwritten
@@ -102,6 +103,21 @@ CASES += [
     (GemmConfig(64, 64, 16, 16, 64, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(70, 92, 52)]),
     (GemmConfig(128, 128, 32, 64, 32, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 300, 72)]),
 ]
+# second operand stored transposed (Bt[N, K]): staged and direct-to-LDS loads, both MFMA shapes, 1, 2 and
+# 4 column blocks per wave (each has its own column permutation), dword path with odd K and N, ragged edges
+CASES += [
+    (GemmConfig(128, 128, 32, 32, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1), [(200, 300, 32), (130, 260, 96), (200, 300, 200), (1, 4, 4)]),
+    (GemmConfig(256, 256, 32, 128, 128, 32, 3, 0, 0, 4, 0, 3, 8, 0, 1, 1), [(512, 512, 64)]),
+    (GemmConfig(256, 256, 32, 64, 128, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1), [(300, 520, 100)]),
+    (GemmConfig(128, 128, 8, 64, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1), [(140, 132, 8), (140, 132, 100)]),
+    (GemmConfig(128, 128, 64, 32, 64, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1), [(200, 300, 136)]),
+    (GemmConfig(128, 128, 32, 64, 32, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1), [(200, 300, 72)]),       # one column block per wave
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 4, 4, 1, 3, 8, 0, 0, 1), [(200, 300, 72), (129, 132, 20)]),
+    (GemmConfig(128, 128, 16, 64, 64, 16, 3, 4, 4, 1, 1, 3, 8, 0, 0, 1), [(37, 53, 29), (130, 127, 17)]),
+    (GemmConfig(64, 64, 16, 16, 64, 16, 1, 4, 4, 1, 1, 3, 8, 0, 0, 1), [(70, 90, 50)]),
+    (GemmConfig(128, 128, 24, 64, 64, 32, 3, 4, 4, 4, 1, 3, 8, 0, 0, 1), [(140, 132, 100)]),
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 0, 0, 4, 0, 3, 8, 0, 0, 1), [(256, 384, 128)]),         # unpadded, aligned
+]
 FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
 
 
@@ -131,6 +147,57 @@ def test_structured_operands_are_exact(device):
     rows = np.random.default_rng(5).integers(0, n, 150)
     pick[np.arange(150), rows] = 1
     assert np.array_equal(run_gemm(cfg, pick, B), B[rows])
+
+
+def test_transposed_second_operand(device):
+    """C = A * Bt^T with Bt[N, ldb >= K]: one-hot operands catch a wrong column permutation, the
+    leading dimension is honoured, the launch checks ldb against K, and the policy -> Compiler path
+    takes the flag at full size (bit-exact on integer inputs, same bits as the B[K, N] kernel)."""
+    cfg = GemmConfig(128, 128, 32, 32, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1)
+    n = 200
+    Bt = np.random.default_rng(3).standard_normal((264, n), dtype=np.float32)           # N x K
+    assert np.array_equal(run_gemm(cfg, np.eye(n, dtype=np.float32), Bt.T), Bt.T)
+    pick = np.zeros((n, 140), np.float32)                                               # B = one-hot columns
+    cols = np.random.default_rng(5).integers(0, n, 140)
+    pick[cols, np.arange(140)] = 1
+    A = np.random.default_rng(4).standard_normal((136, n), dtype=np.float32)
+    assert np.array_equal(run_gemm(cfg, A, pick), A[:, cols])
+
+    M, N, K, ldb = 200, 300, 72, 96
+    rng = np.random.default_rng(21)
+    hA = rng.integers(0, 10, (M, K)).astype(np.float32)
+    hBt = rng.integers(0, 10, (N, ldb)).astype(np.float32)
+    dA, dB, dC = DeviceArray.from_host(hA), DeviceArray.from_host(hBt), DeviceArray((M, N))
+    plan = GemmPlan(cfg)
+    plan.launch(dA, dB, dC, M, N, K, ldb=ldb)
+    hip.synchronize()
+    assert np.array_equal(dC.get(), go.c_gemm_f32(hA, np.ascontiguousarray(hBt[:, :K].T)))
+    with pytest.raises(HipError):
+        plan.launch(dA, dB, dC, M, N, K, ldb=K - 4)
+
+    arch = MI355X.from_device(device)
+    for shape in ((2048, 2048, 2048), (4096, 8192, 4096), (3000, 5000, 1536), (1000, 2002, 514)):
+        mc = MatmulConfig(*shape, 32)
+        hint = get_roller_hints(mc, arch, topk=1)[0]
+        say("trans_b", shape, hint.block_tile, hint.wave_tile, hint.rstep)
+        A, B = go.make_inputs(*shape, seed=2, distribution="integer")
+        dA, dBt, dB = DeviceArray.from_host(A), DeviceArray.from_host(B.T), DeviceArray.from_host(B)
+        outs = []
+        for trans_b, operand in ((True, dBt), (False, dB)):
+            func = roller.Compiler(mc, hint, bm.PIPELINE_DEPTH, trans_b=trans_b).compile()
+            assert func.gemm_config.trans_b == int(trans_b)
+            dC = DeviceArray((shape[0], shape[1]))
+            dC.fill_bytes(0xFF)
+            func(func.grid_dims(), func.block_dims(), (dA, operand, dC))
+            hip.synchronize()
+            outs.append(dC.get())
+        assert np.array_equal(outs[0], go.gemm_f32(A, B)), shape
+        assert np.array_equal(outs[0], outs[1]), shape
+    mc = MatmulConfig(1024, 1024, 512, 32)
+    hint = get_roller_hints(mc, arch, topk=1)[0]
+    func = roller.Compiler(mc, hint, 3, trans_b=True).compile()
+    roller.run_eval(func, 3, hint, repeat_times=3)                  # uniform inputs, tolerance check inside
+    assert func.last_eval["ok"]
 
 
 def test_accumulate_mode_adds_into_c(device):
@@ -388,7 +455,9 @@ def test_run_eval_and_sweep_end_to_end(device, tmp_path, capsys):
     ms, gflops = roller.run_eval(func, 3, hint, repeat_times=5)
     assert ms > 0 and gflops == pytest.approx(2 * 1024 * 1024 * 512 * 1e-9 / (ms / 1e3), rel=1e-6)
     assert func.last_eval["ok"] and func.last_eval["normwise"] <= 1e-5
+    assert 0 < func.last_eval["min_ms"] <= func.last_eval["median_ms"] < 10 * ms
     df = bm.benchmark([(512, 768, 256), (300, 500, 96)], topk=4, csv_path=tmp_path / "r.csv", repeat_times=3)
     assert len(df) == 2 and (tmp_path / "r.csv").exists()
     assert all(df["Best Hint"] != "N/A") and all(df["Normwise Error"] <= 1e-5)
     assert all(df["Max Abs Error"] <= df["Max Abs Bound"])
+    assert all(df["Min Launch (ms)"] <= df["Median Launch (ms)"])
