@@ -22,7 +22,7 @@ from __future__ import annotations
 import itertools
 import math
 from dataclasses import dataclass
-from typing import Iterator, List, Optional
+from typing import Iterator, List, Optional, Sequence
 
 from .arch import CUDA, TileDevice  # noqa: F401  (CUDA re-exported like the reference does)
 from .utils import coalesced_factor, coalesced_tensor_shape, factorize, get_all_factors  # noqa: F401
@@ -236,9 +236,9 @@ class Policy:
     # tile sizes offered in addition to the exact divisors of a dimension
     SIMT_LADDER = (2, 4, 8, 16, 32)
     MFMA_LADDER = (16, 32, 64, 128, 256, 512)
-    # registers per lane the MFMA kernel needs besides its accumulators: two sets of operand
-    # fragments, the global->LDS staging registers and addresses (measured: 90-110)
-    REG_OVERHEAD = 96
+    # registers per lane the MFMA kernel needs besides its accumulators and operand fragments:
+    # addresses, loop state, buffer resources (measured: 40-60)
+    REG_OVERHEAD = 50
 
     def __init__(self, config: MatmulConfig, arch: TileDevice) -> None:
         self.arch = arch
@@ -408,6 +408,19 @@ class Policy:
         td.thread_tile = best
         return td.clone()
 
+    def _reg_overhead(self, td: TileDict, wave_tile: Sequence[int], mi: int, block_size: int) -> int:
+        """Registers per lane besides the accumulators.  The kernel keeps two sets of operand
+        fragments (one 128-bit A value per row block and four B values per column block, i.e.
+        ``4 * (blocks_m + blocks_n)`` registers a set); when its loads cannot go straight to LDS
+        it also stages one K step of both operand tiles in registers."""
+        blocks_m, blocks_n = wave_tile[0] // mi, wave_tile[1] // mi
+        regs = self.REG_OVERHEAD + 2 * 4 * (blocks_m + blocks_n)
+        cfg = self.matmul_config
+        direct = cfg.K % 4 == 0 and cfg.N % 4 == 0 and td.rstep & (td.rstep - 1) == 0
+        if not direct:
+            regs += -(-(sum(td.block_tile) * td.rstep) // block_size)
+        return regs
+
     def _assign_wave_tiles(self, td: TileDict, block_size: int) -> List[TileDict]:
         """The thread-tile step on a device with matrix cores: the block tile is split over
         ``block_size / wave`` wavefronts, once per matrix-instruction shape that admits a split
@@ -433,7 +446,7 @@ class Policy:
             acc_regs = int(math.prod(thread_tile) * self.matmul_config.el_bytes / 4)
             if acc_regs >= arch.thread_reg_limit:
                 continue
-            if budget and acc_regs + self.REG_OVERHEAD > budget:
+            if budget and acc_regs + self._reg_overhead(td, wave_tile, mi, block_size) > budget:
                 continue
             td.thread_tile = thread_tile
             td.wave_tile = wave_tile

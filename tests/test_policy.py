@@ -284,10 +284,11 @@ def test_mi355x_block_sizes_aim_for_two_waves_per_simd():
     assert policy.recommend_block_size(td)[:3] == [512, 256, 1024]      # 8 waves, then 4 and 16 (tie: smaller first)
     assert Policy(cfg, CUDA()).recommend_block_size(TileDict.from_block_tile([128, 128], 32, cfg, CUDA()))[0] == 128
     hints = get_roller_hints(cfg, MI355X(), topk=4)
-    # one block tile, two block sizes, both matrix-instruction shapes
+    # one block tile, two block sizes, both matrix-instruction shapes -- except 16x16x4 at eight
+    # waves, whose 4 x 8 blocks need more fragment registers than half a SIMD's file leaves
     assert [(h.block_tile, h.wave_tile, h.threads, h.mfma) for h in hints] == [
-        ([256, 256], [64, 128], 512, 32), ([256, 256], [64, 128], 512, 16),
-        ([256, 256], [128, 128], 256, 32), ([256, 256], [128, 128], 256, 16)]
+        ([256, 256], [64, 128], 512, 32), ([256, 256], [128, 128], 256, 32),
+        ([256, 256], [128, 128], 256, 16), ([128, 512], [64, 128], 512, 32)]
 
 
 def test_mi355x_register_budget_drops_splits_that_would_spill():
@@ -296,13 +297,16 @@ def test_mi355x_register_budget_drops_splits_that_would_spill():
         for h in get_roller_hints(MatmulConfig(*shape, 32), arch, topk=40):
             waves_per_simd = -(-(h.threads // 64) // arch.sm_partition)
             acc = h.thread_tile[0] * h.thread_tile[1]
-            assert acc + Policy.REG_OVERHEAD <= arch.regs_per_lane // waves_per_simd, h
+            frags = 2 * 4 * (h.wave_tile[0] // h.mfma + h.wave_tile[1] // h.mfma)
+            assert acc + frags + Policy.REG_OVERHEAD <= arch.regs_per_lane // waves_per_simd, h
     cfg = MatmulConfig(8192, 8192, 8192, 32)
     policy = Policy(cfg, arch)
     assert not TileDict.from_block_tile([512, 256], 16, cfg, arch).valid   # 131072 accumulators fill the CU's registers
     td = TileDict.from_block_tile([256, 256], 32, cfg, arch)
-    assert [h.threads for h in policy._assign_wave_tiles(td, 256)] == [256, 256]   # 256 + 96 <= 512
-    assert [h.threads for h in policy._assign_wave_tiles(td, 512)] == [512, 512]   # 128 + 96 <= 256
+    assert [(h.threads, h.mfma) for h in policy._assign_wave_tiles(td, 256)] == [(256, 32), (256, 16)]
+    # eight waves share a SIMD in pairs: 128 accumulators + 48 fragment registers + 50 fit 256,
+    # 128 + 96 + 50 (16x16x4: 4 x 8 blocks) do not -- that kernel spills
+    assert [(h.threads, h.mfma) for h in policy._assign_wave_tiles(td, 512)] == [(512, 32)]
     assert policy._assign_wave_tiles(td, 1024) == []                               # 64 + 96 > 128
     assert policy._assign_wave_tiles(td, 96) == []                                 # not a whole number of waves
 
