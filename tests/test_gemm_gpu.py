@@ -200,6 +200,29 @@ def test_transposed_second_operand(device):
     assert func.last_eval["ok"]
 
 
+def test_seeded_random_shapes_through_policy_are_exact(device):
+    """Forty seeded shapes (ragged, tiny, K and N odd or multiples of 4), each through
+    get_roller_hints -> Compiler at a random pipeline depth, operand layout and accumulate mode:
+    bit-exact against the host GEMM on integer inputs (sums stay far below 2^24)."""
+    from gemm_cases import seeded_policy_cases
+    # the data-sheet model, so that the cases (and the kernels compiled ahead for them) do not depend on the box
+    for case, mc, hint, depth, trans_b, accumulate in seeded_policy_cases(MI355X()):
+        M, N, K = mc.M, mc.N, mc.K
+        say("random case", case, (M, N, K), "depth", depth, "trans_b", trans_b, "accumulate", accumulate,
+            hint.block_tile, hint.wave_tile, hint.rstep)
+        func = roller.Compiler(mc, hint, depth, accumulate=accumulate, trans_b=trans_b).compile()
+        rng = np.random.default_rng(1000 + case)
+        A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+        B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+        C0 = rng.integers(-50, 50, (M, N)).astype(np.float32)
+        dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B.T if trans_b else B)
+        dC = DeviceArray.from_host(C0)
+        func(func.grid_dims(), func.block_dims(), (dA, dB, dC))
+        hip.synchronize()
+        want = A @ B + (C0 if accumulate else 0)
+        assert np.array_equal(dC.get(), want), (case, M, N, K, func.gemm_config.tag())
+
+
 def test_accumulate_mode_adds_into_c(device):
     M, N, K = 300, 260, 100
     A, B = go.make_inputs(M, N, K, seed=11, distribution="integer")
