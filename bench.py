@@ -1,7 +1,7 @@
 """Headline benchmark: fp32 GEMM TFLOP/s of the Roller-selected HIP kernels over M0..M13 on one
 MI355X, as one JSON line on stdout (everything else goes to stderr).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sweep|M0..M13|cfg4] [--topk 20]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload sweep|M0..M13|cfg4|MxNxK] [--topk 20]
 
 A "step" is one pass over the workload: one launch of the best kernel for every shape in it,
 with A, B and C resident in HBM.  Before the timed region, and reported separately, the Roller
@@ -107,7 +107,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="sweep", help="sweep (M0..M13), one of M0..M13, cfg4 (3000x5000x1536), or copy (traffic-counter calibration)")
+    ap.add_argument("--workload", default="sweep", help="sweep (M0..M13), one of M0..M13, cfg4 (3000x5000x1536), any MxNxK, or copy (traffic-counter calibration)")
     ap.add_argument("--topk", type=int, default=20)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--retune", action="store_true", help="ignore remembered winners")
@@ -136,6 +136,13 @@ def main() -> int:
     elif args.workload == "cfg4":
         names, shapes = ["cfg4"], [(3000, 5000, 1536)]
         workload = "cfg4: M=3000 N=5000 K=1536, standard-normal entries (ragged tiles)"
+    elif "x" in args.workload:
+        dims = tuple(int(v) for v in args.workload.lower().split("x"))
+        if len(dims) != 3 or min(dims) <= 0:
+            print(f"bench.py: --workload {args.workload}: expected MxNxK", file=sys.stderr)
+            return 2
+        names, shapes = [args.workload.lower()], [dims]
+        workload = f"M={dims[0]} N={dims[1]} K={dims[2]}"
     else:
         idx = int(args.workload.lstrip("Mm"))
         names, shapes = [f"M{idx}"], [README_SHAPES[idx]]

@@ -7,7 +7,9 @@ try/except so that one failing hint never ends the sweep (:41-58), a summary tab
 written to ``benchmark_results.csv`` (:89-95).  The table keeps the reference's columns (the
 baseline is numpy's BLAS on the host cores instead of CuPy/cuBLAS, so the two "CuPy" columns
 are named "Host") and adds what an MI355X run is judged by: TFLOP/s, % of the fp32-matrix peak,
-policy-search and JIT time, the rank of the winning hint, and the error measures.
+policy-search and JIT time, the rank of the winning hint, the error measures and, with
+``counters=True`` / ``--counters``, what rocprofv3 counts for the winning kernel: MFMA busy %,
+LDS bank conflicts, HBM-side GB/s and traffic over algorithmic bytes.
 """
 
 from __future__ import annotations
@@ -40,10 +42,11 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
               arch: Optional[TileDevice] = None, baseline: bool = True,
               csv_path: Optional[os.PathLike] = "benchmark_results.csv",
               dump_path: Optional[os.PathLike] = None, repeat_times: int = 20,
-              distribution: str = "uniform", seed: int = 0) -> pd.DataFrame:
+              distribution: str = "uniform", seed: int = 0, counters: bool = False) -> pd.DataFrame:
     arch = arch or MI355X()
     peak_tflops = arch.peak_matrix_tflops or float("nan")
     results = []
+    counter_rows = collect_counters(test_shapes) if counters else {}
 
     for m, n, k in test_shapes:
         print(f"--- Benchmarking M={m}, N={n}, K={k} ---")
@@ -120,6 +123,7 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
             "Normwise Error": best_info.get("normwise", float("nan")),
             "Max Abs Error": best_info.get("max_abs", float("nan")),
             "Max Abs Bound": best_info.get("bound", float("nan")),
+            **counter_rows.get((m, n, k), {}),
         })
         print("-" * 50)
 
@@ -131,6 +135,32 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
         df.to_csv(csv_path, index=False)
         print(f"\nResults saved to {csv_path}")
     return df
+
+
+COUNTER_COLUMNS = ("MfmaUtil %", "LdsBankConflict", "HBM-side GB/s", "Traffic / algorithmic", "MFMA FLOP / 2MNK")
+
+
+def collect_counters(test_shapes: Sequence[Tuple[int, int, int]]) -> dict:
+    """rocprofv3 counters per shape (MFMA busy %, LDS bank conflicts, HBM-side GB/s) as extra table
+    columns.  The profiled runs are child processes and must be started before this process
+    creates its own GPU context, which is why the sweep collects them first."""
+    import shutil
+    import tempfile
+
+    from . import counters as pmc
+    from . import hip
+
+    if hip._initialised:
+        raise RuntimeError("counters must be collected before this process initialises the GPU")
+    if shutil.which("rocprofv3") is None:
+        raise RuntimeError("rocprofv3 not found on PATH")
+    names = [pmc.workload_name(s) for s in test_shapes]
+    work = Path(tempfile.mkdtemp(prefix="roller_counters_", dir="/tmp"))
+    try:
+        rows = pmc.collect(names, work)
+    finally:
+        shutil.rmtree(work, ignore_errors=True)
+    return {(r["M"], r["N"], r["K"]): {c: r[c] for c in COUNTER_COLUMNS if c in r} for r in rows}
 
 
 def plot_results(df: pd.DataFrame, path: os.PathLike, peak_tflops: float = 157.3) -> Path:
@@ -169,13 +199,16 @@ def main(argv=None) -> None:
     ap.add_argument("--csv", default="benchmark_results.csv")
     ap.add_argument("--dump", default=None, help="directory for kernel source / ISA dumps")
     ap.add_argument("--plot", default=None, help="write a bar chart of the sweep to this image file")
+    ap.add_argument("--counters", action="store_true",
+                    help="add rocprofv3 counter columns (MFMA busy %%, LDS bank conflicts, HBM-side GB/s); several extra runs per shape")
     args = ap.parse_args(argv)
     if args.shapes == "full":
         dims = [2048, 4096, 8192]
         shapes = list(itertools.product(dims, dims, dims))
     else:
         shapes = README_SHAPES
-    df = benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump)
+    df = benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump,
+                   counters=args.counters)
     if args.plot:
         print(f"Chart saved to {plot_results(df, args.plot)}")
 

@@ -48,6 +48,25 @@ SHAPES = {f"M{i}": s for i, s in enumerate([
 SHAPES["cfg4"] = (3000, 5000, 1536)
 
 
+def shape_of(name: str):
+    """(M, N, K) of a workload name: M0..M13, cfg4, or a literal ``MxNxK``."""
+    if name in SHAPES:
+        return SHAPES[name]
+    dims = tuple(int(v) for v in name.lower().split("x"))
+    if len(dims) != 3 or min(dims) <= 0:
+        raise ValueError(f"unknown workload {name!r}")
+    return dims
+
+
+def workload_name(shape) -> str:
+    """The shortest name ``bench.py --workload`` accepts for a shape."""
+    shape = tuple(int(v) for v in shape)
+    for name, known in SHAPES.items():
+        if known == shape:
+            return name
+    return "x".join(str(v) for v in shape)
+
+
 def _run(cmd: List[str], cwd: Path, timeout: int) -> subprocess.CompletedProcess:
     env = dict(os.environ, TMPDIR=str(cwd))
     return subprocess.run(cmd, cwd=str(cwd), env=env, capture_output=True, text=True, timeout=timeout)
@@ -129,7 +148,7 @@ def collect(shape_names: List[str], work: Path, verbose: bool = True) -> List[Di
     say(f"[counters] scale factors: FETCH_SIZE x{fetch_scale:.3f}, WRITE_SIZE x{write_scale:.3f}")
     rows = []
     for name in shape_names:
-        shape = SHAPES[name]
+        shape = shape_of(name)
         plain = profiled_bench(name, None, work, f"plain_{name}")["bench"]
         ms = plain["per_shape"][0]["ms"]
         merged: Dict[str, float] = {}
@@ -146,16 +165,18 @@ def collect(shape_names: List[str], work: Path, verbose: bool = True) -> List[Di
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description="rocprofv3 counters for the Roller-selected GEMM kernels")
-    ap.add_argument("--shapes", nargs="*", default=["M0", "M10"], help="M0..M13, cfg4 (default: M0 M10)")
+    ap.add_argument("--shapes", nargs="*", default=["M0", "M10"], help="M0..M13, cfg4 or MxNxK (default: M0 M10)")
     ap.add_argument("--csv", default="gemm_counters.csv")
     ap.add_argument("--keep", action="store_true", help="keep the rocprofv3 output directory")
     args = ap.parse_args(argv)
     if shutil.which("rocprofv3") is None:
         print("rocprofv3 not found on PATH", file=sys.stderr)
         return 2
-    unknown = [s for s in args.shapes if s not in SHAPES]
-    if unknown:
-        print(f"unknown shapes: {unknown}", file=sys.stderr)
+    try:
+        for s in args.shapes:
+            shape_of(s)
+    except ValueError as e:
+        print(e, file=sys.stderr)
         return 2
     work = Path(tempfile.mkdtemp(prefix="roller_counters_", dir="/tmp"))
     try:

@@ -48,3 +48,14 @@ def test_counter_groups_respect_the_per_run_limits():
         assert sum(n.startswith("GRBM_") for n in names) <= 2
         assert not ({"FETCH_SIZE", "WRITE_SIZE"} <= set(names))     # 3 + 2 TCC counters exceed the 4 available
     assert counters.SHAPES["M10"] == (4096, 8192, 4096) and len(counters.SHAPES) == 15
+
+
+def test_workload_names_round_trip():
+    assert counters.shape_of("M10") == (4096, 8192, 4096) and counters.shape_of("cfg4") == (3000, 5000, 1536)
+    assert counters.shape_of("300x500x96") == (300, 500, 96)
+    assert counters.workload_name((4096, 8192, 4096)) == "M10"
+    assert counters.workload_name((300, 500, 96)) == "300x500x96"
+    assert counters.shape_of(counters.workload_name((7, 8, 9))) == (7, 8, 9)
+    for bad in ("M99", "3x4", "0x4x4", "axbxc"):
+        with pytest.raises(ValueError):
+            counters.shape_of(bad)

@@ -123,6 +123,38 @@ def test_sweep_survives_failing_hints(monkeypatch, tmp_path):
         assert col in df.columns
 
 
+def test_sweep_merges_counter_columns_and_collects_them_first(monkeypatch):
+    order = []
+
+    class FakeCompiler:
+        def __init__(self, config, hint, depth, dump_path=None):
+            self.hint = hint
+
+        def compile(self):
+            order.append("compile")
+            return _FakeFunc(self.hint)
+
+    def fake_collect(shapes):
+        order.append("counters")
+        return {tuple(s): {"MfmaUtil %": 95.0, "LdsBankConflict": 0.0, "HBM-side GB/s": 510.0} for s in shapes}
+
+    monkeypatch.setattr(bm, "Compiler", FakeCompiler)
+    monkeypatch.setattr(bm, "run_eval", lambda func, depth, hint, **k: (1.0, 1000.0))
+    monkeypatch.setattr(bm, "collect_counters", fake_collect)
+    df = bm.benchmark([(2048, 2048, 2048)], topk=2, baseline=False, csv_path=None, counters=True)
+    assert order[0] == "counters" and "compile" in order           # profiled child runs come before any GPU work here
+    assert df.iloc[0]["MfmaUtil %"] == 95.0 and df.iloc[0]["LdsBankConflict"] == 0.0 and df.iloc[0]["HBM-side GB/s"] == 510.0
+    plain = bm.benchmark([(2048, 2048, 2048)], topk=1, baseline=False, csv_path=None)
+    assert "MfmaUtil %" not in plain.columns
+
+
+def test_counter_collection_refuses_an_initialised_process(monkeypatch):
+    from mlir_roller_amd import hip
+    monkeypatch.setattr(hip, "_initialised", True)
+    with pytest.raises(RuntimeError, match="before this process initialises the GPU"):
+        bm.collect_counters([(2048, 2048, 2048)])
+
+
 def test_sweep_reports_all_failed(monkeypatch):
     class AlwaysFails:
         def __init__(self, *a, **k):
