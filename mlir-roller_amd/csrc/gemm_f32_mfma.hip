@@ -12,7 +12,8 @@
 // buffers (the reference's pipeline_depth), accumulators held in registers across the K loop and
 // written once, and a workgroup-id remap for cache reuse (the reference swizzles in panels of 8,
 // roller.py:334-339).  What differs is everything below that level: the per-thread outer product
-// becomes a per-wave grid of MFMA blocks, and cp.async becomes register-staged prefetch.
+// becomes a per-wave grid of MFMA blocks, and cp.async becomes buffer loads that write LDS directly
+// (DIRECT) or a register-staged prefetch.
 //
 // Parameters (all compile-time):
 //   BM, BN      block tile (rows, columns of C per workgroup)
