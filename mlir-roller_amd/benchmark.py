@@ -5,8 +5,9 @@ Same entry point and flow as /root/reference/src/benchmark.py:10-95 -- ``benchma
 topk=20)``, per-shape baseline inside try/except (:19-26), per-hint compile + eval inside
 try/except so that one failing hint never ends the sweep (:41-58), a summary table printed and
 written to ``benchmark_results.csv`` (:89-95).  The table keeps the reference's columns (the
-baseline is numpy's BLAS on the host cores instead of CuPy/cuBLAS, so the two "CuPy" columns
-are named "Host") and adds what an MI355X run is judged by: TFLOP/s, % of the fp32-matrix peak,
+baseline is numpy's BLAS on the host cores, so the two "CuPy" columns are named "Host"; with
+``vendor=True`` / ``--vendor`` rocBLAS sgemm on the GPU is timed as well, the counterpart of the
+reference's cuBLAS column) and adds what an MI355X run is judged by: TFLOP/s, % of the fp32-matrix peak,
 policy-search and JIT time, the rank of the winning hint, the error measures and, with
 ``counters=True`` / ``--counters``, what rocprofv3 counts for the winning kernel: MFMA busy %,
 LDS bank conflicts, HBM-side GB/s and traffic over algorithmic bytes.
@@ -25,7 +26,7 @@ import pandas as pd
 
 from .analyze import MatmulConfig, get_roller_hints
 from .arch import MI355X, TileDevice
-from .roller import Compiler, run_baseline, run_eval
+from .roller import Compiler, run_baseline, run_eval, run_vendor_baseline
 
 PIPELINE_DEPTH = 3
 
@@ -42,7 +43,8 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
               arch: Optional[TileDevice] = None, baseline: bool = True,
               csv_path: Optional[os.PathLike] = "benchmark_results.csv",
               dump_path: Optional[os.PathLike] = None, repeat_times: int = 20,
-              distribution: str = "uniform", seed: int = 0, counters: bool = False) -> pd.DataFrame:
+              distribution: str = "uniform", seed: int = 0, counters: bool = False,
+              vendor: bool = False) -> pd.DataFrame:
     arch = arch or MI355X()
     peak_tflops = arch.peak_matrix_tflops or float("nan")
     results = []
@@ -62,6 +64,17 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
             except Exception as e:
                 print(f"Host baseline failed: {e}")
                 baseline_time, baseline_gflops = float("inf"), 0
+
+        # 1b. vendor BLAS on the GPU: the reference's cuBLAS column (benchmark.py:19-26)
+        vendor_time, vendor_gflops = float("inf"), 0
+        if vendor:
+            print("Running rocBLAS sgemm baseline...")
+            try:
+                vendor_time, vendor_gflops = run_vendor_baseline(config, seed=seed)
+                print(f"rocBLAS baseline: {vendor_time:.6f} ms, {vendor_gflops:.6f} GFLOPS")
+            except Exception as e:
+                print(f"rocBLAS baseline failed: {e}")
+                vendor_time, vendor_gflops = float("inf"), 0
 
         # 2. roller hints
         # the reference runs depth 2 (benchmark.py:29); here 3 = two LDS buffers + a register stage
@@ -110,6 +123,9 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
             "Roller GFLOPS": best_gflops,
             "Speedup vs Host": (baseline_time / best_time
                                 if best_time > 0 and baseline_time != float("inf") else 0),
+            **({"rocBLAS Time (ms)": vendor_time, "rocBLAS GFLOPS": vendor_gflops,
+                "Speedup vs rocBLAS": (vendor_time / best_time
+                                       if best_time > 0 and vendor_time != float("inf") else 0)} if vendor else {}),
             "Best Hint": str(best_hint) if best_hint else "N/A",
             "Roller TFLOPS": tflops,
             "% of fp32 matrix peak": 100.0 * tflops / peak_tflops,
@@ -179,9 +195,12 @@ def plot_results(df: pd.DataFrame, path: os.PathLike, peak_tflops: float = 157.3
     ax.axhline(100.0, color="black", linewidth=0.8, linestyle="--")
     ax.set_ylim(0, 110)
     ax.set_ylabel(f"% of fp32 matrix peak ({peak_tflops:g} TFLOP/s)")
-    ax.set_title("GEMM FP32 on MI355X (Roller-selected HIP MFMA kernels)")
-    for bar, tf, sp in zip(bars, df["Roller TFLOPS"], df["Speedup vs Host"]):
-        text = f"{tf:.0f}" + (f"\n{sp:.0f}x host" if sp else "")
+    ax.set_title("GEMM FP32 on MI355X (Roller-selected HIP MFMA kernels)"
+                 + ("\nabove each bar: TFLOP/s and speed relative to rocBLAS sgemm" if "Speedup vs rocBLAS" in df.columns else ""),
+                 fontsize=10)
+    vendor = df["Speedup vs rocBLAS"] if "Speedup vs rocBLAS" in df.columns else [0] * len(df)
+    for bar, tf, sp, sv in zip(bars, df["Roller TFLOPS"], df["Speedup vs Host"], vendor):
+        text = f"{tf:.0f}" + (f"\n{sv:.2f}x" if sv else (f"\n{sp:.0f}x host" if sp else ""))
         ax.text(bar.get_x() + bar.get_width() / 2, bar.get_height() + 1, text, ha="center", va="bottom", fontsize=7)
     fig.tight_layout()
     out = Path(path)
@@ -199,6 +218,7 @@ def main(argv=None) -> None:
     ap.add_argument("--csv", default="benchmark_results.csv")
     ap.add_argument("--dump", default=None, help="directory for kernel source / ISA dumps")
     ap.add_argument("--plot", default=None, help="write a bar chart of the sweep to this image file")
+    ap.add_argument("--vendor", action="store_true", help="also time rocBLAS sgemm on the GPU (the reference's cuBLAS column)")
     ap.add_argument("--counters", action="store_true",
                     help="add rocprofv3 counter columns (MFMA busy %%, LDS bank conflicts, HBM-side GB/s); several extra runs per shape")
     args = ap.parse_args(argv)
@@ -208,7 +228,7 @@ def main(argv=None) -> None:
     else:
         shapes = README_SHAPES
     df = benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump,
-                   counters=args.counters)
+                   counters=args.counters, vendor=args.vendor)
     if args.plot:
         print(f"Chart saved to {plot_results(df, args.plot)}")
 

@@ -339,6 +339,36 @@ def run_baseline(config: MatmulConfig, repeat_times: int = 3, seed: int = 0):
     return best * 1e3, gflops
 
 
+def run_vendor_baseline(config: MatmulConfig, repeat_times: int = 50, seed: int = 0, check: bool = True):
+    """The reference's baseline proper (roller.py:589-607): the vendor BLAS on the GPU -- there
+    cuBLAS through ``cp.matmul``, here rocBLAS ``sgemm`` -- on the same seeded inputs, timed like
+    the kernels (clock ramp queued ahead, ``repeat_times`` launches between two events).
+    Returns ``(ms, gflops)``; raises if rocBLAS is missing or its result is outside the tolerances."""
+    from .vendor_blas import rocblas
+
+    M, N, K = config.M, config.N, config.K
+    case = _host_case(config, seed, "uniform")
+    A, B, C32 = case[0], case[1], case[2]
+    dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray.zeros((M, N))
+    blas = rocblas()
+    blas.sgemm_row_major(dA, dB, dC, M, N, K)
+    hip.synchronize()
+    if check:
+        info = gemm_errors(dC.get(), A, B, C32, _host_case_f64(case))
+        if not info["ok"]:
+            raise AssertionError(f"rocBLAS result outside tolerance: {info}")
+    est_ms = 2.0 * M * N * K / 120e9
+    for _ in range(max(10, int(WARMUP_MS / est_ms) + 1)):
+        blas.sgemm_row_major(dA, dB, dC, M, N, K)
+    with time_cuda() as (start_gpu, end_gpu):
+        for _ in range(repeat_times):
+            blas.sgemm_row_major(dA, dB, dC, M, N, K)
+    t = hip.get_elapsed_time(start_gpu, end_gpu) / repeat_times
+    gflops = 2 * M * N * K * 1e-9 / (t / 1000)
+    print(f"t={t:.6f} ms GFLOPS={gflops:.6f}")
+    return t, gflops
+
+
 if __name__ == "__main__":
     S = 4096
     config = MatmulConfig(M=S, N=S, K=S, el_bits=32)

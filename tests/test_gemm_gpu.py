@@ -457,6 +457,21 @@ def test_operands_larger_than_4_gib(device, which, shape, cfg):
         assert np.array_equal(got[r0:r0 + 4096], want[r0:r0 + 4096]), (which, r0)
 
 
+def test_vendor_baseline_is_a_correct_row_major_gemm(device):
+    """The rocBLAS column of the sweep: the column-major call really computes row-major A @ B
+    (non-square, so that a swapped operand or dimension shows), and the timing helper checks it."""
+    from mlir_roller_amd.vendor_blas import rocblas
+    M, N, K = 200, 304, 72
+    A, B = go.make_inputs(M, N, K, seed=9, distribution="integer")
+    dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray((M, N))
+    dC.fill_bytes(0xFF)
+    rocblas().sgemm_row_major(dA, dB, dC, M, N, K)
+    hip.synchronize()
+    assert np.array_equal(dC.get(), go.gemm_f32(A, B))
+    ms, gflops = roller.run_vendor_baseline(MatmulConfig(512, 768, 256, 32), repeat_times=3)
+    assert ms > 0 and gflops == pytest.approx(2 * 512 * 768 * 256 * 1e-9 / (ms / 1e3), rel=1e-6)
+
+
 def test_handle_checks_grid_and_block(device):
     cfg = MatmulConfig(512, 512, 128, 32)
     hint = get_roller_hints(cfg, MI355X(), topk=1)[0]

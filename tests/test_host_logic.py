@@ -155,6 +155,29 @@ def test_counter_collection_refuses_an_initialised_process(monkeypatch):
         bm.collect_counters([(2048, 2048, 2048)])
 
 
+def test_sweep_vendor_columns(monkeypatch):
+    class FakeCompiler:
+        def __init__(self, config, hint, depth, dump_path=None):
+            self.hint = hint
+
+        def compile(self):
+            return _FakeFunc(self.hint)
+
+    monkeypatch.setattr(bm, "Compiler", FakeCompiler)
+    monkeypatch.setattr(bm, "run_eval", lambda func, depth, hint, **k: (2.0, 1000.0))
+    monkeypatch.setattr(bm, "run_vendor_baseline", lambda config, seed=0: (3.0, 700.0))
+    df = bm.benchmark([(2048, 2048, 2048)], topk=1, baseline=False, csv_path=None, vendor=True)
+    r = df.iloc[0]
+    assert r["rocBLAS Time (ms)"] == 3.0 and r["rocBLAS GFLOPS"] == 700.0 and r["Speedup vs rocBLAS"] == pytest.approx(1.5)
+
+    def broken(config, seed=0):
+        raise OSError("librocblas.so missing")
+    monkeypatch.setattr(bm, "run_vendor_baseline", broken)          # a missing library never ends the sweep
+    r = bm.benchmark([(2048, 2048, 2048)], topk=1, baseline=False, csv_path=None, vendor=True).iloc[0]
+    assert r["rocBLAS Time (ms)"] == float("inf") and r["Speedup vs rocBLAS"] == 0
+    assert "rocBLAS GFLOPS" not in bm.benchmark([(2048, 2048, 2048)], topk=1, baseline=False, csv_path=None).columns
+
+
 def test_sweep_reports_all_failed(monkeypatch):
     class AlwaysFails:
         def __init__(self, *a, **k):
