@@ -262,6 +262,18 @@ DEV int bt_col_of_row(int row) {
 }
 #endif
 
+// The same with STRIDE MFMAs ahead of each of the NO other instructions (needs NO * STRIDE <= NM).
+template <int NM, int NO, int MASK, int STRIDE>
+DEV void stride_with_mfma() {
+  static_assert(NO * STRIDE <= NM, "not enough MFMAs for this spacing");
+#pragma unroll
+  for (int i = 0; i < NO; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, STRIDE, 0);
+    __builtin_amdgcn_sched_group_barrier(MASK, 1, 0);
+  }
+  if constexpr (NM - NO * STRIDE > 0) __builtin_amdgcn_sched_group_barrier(0x008, NM - NO * STRIDE, 0);
+}
+
 // Maps the hardware workgroup id to a tile of C.
 DEV bool tile_of_workgroup(int nbm, int nbn, int& tile_m, int& tile_n) {
   int pid = blockIdx.y * gridDim.x + blockIdx.x;
@@ -560,8 +572,10 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       }
       // the last round is split around the barrier: its first half covers the LDS writes of
       // tile kt+1 and the global loads of tile kt+2, its second half the first reads of tile kt+1
-      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
+      // (DIRECT: one quarter before the barrier, three after it, which leaves room to issue the
+      // loads of tile kt+2 behind every second MFMA instead of every one: measured 0.3-0.8 % faster)
 #if DIRECT
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 1);
       // Tile kt+1 was requested one step ago, straight into the other buffer; once every wave's
       // part has landed and all have met, buffer `cur` is free again and takes tile kt+2.
 #if SCHED
@@ -572,12 +586,20 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       __syncthreads();
       read_frags(fr[(P + SUPERS) & 1], cur ^ 1, 0);
       fetch_direct(kt + 2, cur);
-      mfma_frags(fr[(P + SUPERS - 1) & 1], 2, 4);
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 1, 4);
 #if SCHED
-      interleave_with_mfma<G / 4, R, 0x100>();
-      interleave_with_mfma<G / 2 - G / 4, L, 0x020>();
+      {
+        constexpr int REST = 3 * G / 4, PAIRED = R < REST ? R : REST, LEFT = REST - PAIRED;
+        interleave_with_mfma<PAIRED, R, 0x100>();
+        if constexpr (LEFT >= 2 * L) {
+          stride_with_mfma<LEFT, L, 0x020, 2>();
+        } else {
+          interleave_with_mfma<LEFT, L, 0x020>();
+        }
+      }
 #endif
 #else
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
       stash(cur ^ 1);
       fetch(kt + 2);
 #if SCHED
