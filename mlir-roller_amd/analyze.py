@@ -200,11 +200,18 @@ def _similarity(a: float, b: float) -> float:
     return (2 * a * b) / (a * a + b * b)
 
 
+# MFMA blocks one wave may own: the kernel keeps one accumulator vector per block in an array that
+# the compiler holds in registers only up to this many (128x128 with the 16x16x4 shape, 64 blocks,
+# ends up in scratch memory and runs 50x slower)
+MAX_BLOCKS_PER_WAVE = 32
+
+
 def split_block_over_waves(block_tile: List[int], waves: int, rstep: int, arch: TileDevice, shapes=None):
     """Wave tile ``[wm, wn]`` and MFMA size for a block tile computed by ``waves`` wavefronts,
     or None.  A wave tile must be a grid of MFMA blocks whose column count the kernel reads
     with one vector load (1, 2 or a multiple of 4 blocks), and the reduce step must hold whole
-    128-bit fragment reads (4 * wave / mi elements of k).  The larger instruction is preferred;
+    128-bit fragment reads (4 * wave / mi elements of k), and a wave owns at most
+    ``MAX_BLOCKS_PER_WAVE`` blocks.  The larger instruction is preferred;
     among its wave tiles the most square wins, wider before taller."""
     m, n = block_tile
     for shape in (arch.mfma_shapes if shapes is None else shapes):
@@ -221,6 +228,8 @@ def split_block_over_waves(block_tile: List[int], waves: int, rstep: int, arch: 
                 continue
             col_blocks = wn // mi
             if not (col_blocks in (1, 2) or col_blocks % 4 == 0):
+                continue
+            if (wm // mi) * col_blocks > MAX_BLOCKS_PER_WAVE:
                 continue
             key = (wm + wn, -wn)
             if best is None or key < best[0]:

@@ -163,6 +163,7 @@ static_assert(MI == 32 || MI == 16, "MI selects v_mfma_f32_32x32x2_f32 or v_mfma
 static_assert(BM % WM == 0 && BN % WN == 0, "wave tile must divide block tile");
 static_assert(WM % MI == 0 && WN % MI == 0, "MFMA block must divide wave tile");
 static_assert(TN == 1 || TN == 2 || TN % 4 == 0, "column blocks per wave: 1, 2 or a multiple of 4");
+static_assert(TM * TN <= 32, "at most 32 MFMA blocks per wave: beyond that the accumulator array is no longer kept in registers");
 static_assert(BK % KSUPER == 0, "BK must be a multiple of 4*(64/MI)");
 static_assert(PAD_A % 4 == 0 && PAD_B % 4 == 0, "LDS rows stay 16-byte aligned");
 static_assert(TRANS_B == 0 || TRANS_B == 1, "TRANS_B is a flag");

@@ -354,6 +354,35 @@ def compile_source(source: str, name: str = "kernel.hip", options: Sequence[str]
     return blob, text
 
 
+def code_object_resources(code: bytes) -> dict:
+    """Register, spill and scratch figures from the metadata note of a gfx950 code object (the same
+    msgpack keys ``rl_gemm_plan_resources`` reads); -1 where a key is missing.  Needs no GPU."""
+    def value_after(key: bytes) -> int:
+        i = code.find(key)
+        if i < 0 or i + len(key) >= len(code):
+            return -1
+        p = code[i + len(key):i + len(key) + 5]
+        if p[0] <= 0x7F:
+            return p[0]
+        if p[0] == 0xCC and len(p) >= 2:
+            return p[1]
+        if p[0] == 0xCD and len(p) >= 3:
+            return (p[1] << 8) | p[2]
+        if p[0] == 0xCE and len(p) >= 5:
+            return int.from_bytes(p[1:5], "big")
+        return -1
+    names = {"vgprs": b".vgpr_count", "agprs": b".agpr_count", "sgprs": b".sgpr_count",
+             "vgpr_spills": b".vgpr_spill_count", "sgpr_spills": b".sgpr_spill_count",
+             "scratch_bytes": b".private_segment_fixed_size"}
+    return {k: value_after(v) for k, v in names.items()}
+
+
+def compile_config(cfg: "GemmConfig") -> bytes:
+    """The kernel template compiled for ``cfg`` through hiprtc, without cache or GPU."""
+    options = [f"-D{f.name.upper()}={getattr(cfg, f.name)}" for f in fields(cfg)]
+    return compile_source(template_source(), "gemm_f32_mfma.hip", options)[0]
+
+
 class Module:
     """Counterpart of ``cp.cuda.Module`` (roller.py:504-506)."""
 

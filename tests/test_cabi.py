@@ -88,6 +88,14 @@ def test_config_check_rejects(hip_lib, bad, needle):
     assert err.value.status == hip.RL_ERR_INVALID_ARG and needle in str(err.value)
 
 
+def test_config_check_limits_mfma_blocks_per_wave(hip_lib):
+    hip.config_check(GemmConfig(256, 128, 32, 128, 64, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1))        # 8 x 4 blocks
+    with pytest.raises(HipError, match="at most 32"):
+        hip.config_check(GemmConfig(256, 256, 32, 128, 128, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1))   # 8 x 8 blocks
+    with pytest.raises(HipError, match="32 MFMA blocks"):
+        hip.compile_source(hip.template_source(), "gemm.hip", ["-DBM=256", "-DBN=256", "-DWM=128", "-DWN=128", "-DMI=16", "-DBK=32"])
+
+
 def test_compile_plain_source_without_gpu(hip_lib):
     code, log = hip.compile_source('extern "C" __global__ void k(float* p) { p[threadIdx.x] = 1.0f; }', "k.hip")
     assert code[:4] == b"\x7fELF" and len(code) > 1000

@@ -284,11 +284,14 @@ def test_mi355x_block_sizes_aim_for_two_waves_per_simd():
     assert policy.recommend_block_size(td)[:3] == [512, 256, 1024]      # 8 waves, then 4 and 16 (tie: smaller first)
     assert Policy(cfg, CUDA()).recommend_block_size(TileDict.from_block_tile([128, 128], 32, cfg, CUDA()))[0] == 128
     hints = get_roller_hints(cfg, MI355X(), topk=4)
-    # one block tile, two block sizes, both matrix-instruction shapes -- except 16x16x4 at eight
-    # waves, whose 4 x 8 blocks need more fragment registers than half a SIMD's file leaves
+    # one block tile at two block sizes, then the next tile.  The 16x16x4 shape is out for both: at
+    # eight waves its 4 x 8 blocks need more fragment registers than half a SIMD's file leaves, at
+    # four waves 128x128 would be 64 blocks, more than the kernel keeps in registers
     assert [(h.block_tile, h.wave_tile, h.threads, h.mfma) for h in hints] == [
         ([256, 256], [64, 128], 512, 32), ([256, 256], [128, 128], 256, 32),
-        ([256, 256], [128, 128], 256, 16), ([128, 512], [64, 128], 512, 32)]
+        ([128, 512], [64, 128], 512, 32), ([128, 512], [128, 128], 256, 32)]
+    assert analyze.split_block_over_waves([256, 256], 4, 32, MI355X(), shapes=[(16, 16, 4)]) is None
+    assert analyze.split_block_over_waves([256, 128], 4, 32, MI355X(), shapes=[(16, 16, 4)]) == ([64, 128], 16)   # 4 x 8 = 32 blocks
 
 
 def test_mi355x_register_budget_drops_splits_that_would_spill():
@@ -303,7 +306,7 @@ def test_mi355x_register_budget_drops_splits_that_would_spill():
     policy = Policy(cfg, arch)
     assert not TileDict.from_block_tile([512, 256], 16, cfg, arch).valid   # 131072 accumulators fill the CU's registers
     td = TileDict.from_block_tile([256, 256], 32, cfg, arch)
-    assert [(h.threads, h.mfma) for h in policy._assign_wave_tiles(td, 256)] == [(256, 32), (256, 16)]
+    assert [(h.threads, h.mfma) for h in policy._assign_wave_tiles(td, 256)] == [(256, 32)]
     # eight waves share a SIMD in pairs: 128 accumulators + 48 fragment registers + 50 fit 256,
     # 128 + 96 + 50 (16x16x4: 4 x 8 blocks) do not -- that kernel spills
     assert [(h.threads, h.mfma) for h in policy._assign_wave_tiles(td, 512)] == [(512, 32)]
@@ -322,3 +325,20 @@ def test_mi355x_reduce_step_grows_when_the_grid_leaves_room():
     td = TileDict.from_block_tile([128, 128], 32, cfg, arch)
     policy._expand_reduce_axis(td)
     assert td.rstep == 32
+
+
+def test_mi355x_top_hints_compile_without_spills_or_scratch():
+    """The register model against the real compiler: the first eight hints of every benchmark shape
+    (and of two ragged ones) become kernels that spill nothing and use no scratch memory."""
+    from mlir_roller_amd import hip
+    from mlir_roller_amd.benchmark import README_SHAPES
+    seen = {}
+    for shape in list(README_SHAPES) + [(3000, 5000, 1536), (200, 300, 72)]:
+        cfg = MatmulConfig(*shape, 32)
+        for h in get_roller_hints(cfg, MI355X(), topk=8):
+            seen.setdefault(hint_to_gemm_config(cfg, h, 3), (shape, h))
+    assert len(seen) >= 20
+    for g, (shape, h) in seen.items():
+        res = hip.code_object_resources(hip.compile_config(g))
+        assert res["vgpr_spills"] == 0 and res["sgpr_spills"] == 0 and res["scratch_bytes"] == 0, (shape, g.tag(), res)
+        assert 0 < res["vgprs"] <= 512 // max(1, g.threads // 256), (g.tag(), res)
