@@ -42,7 +42,7 @@ PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix peak: 256 CUs * 256 FLOP/clk * 2
 # measured offline with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE in separate runs and scaled by
 # what the same counters read for a 256 MiB copy kernel (FETCH_SIZE x2.0, WRITE_SIZE x1.0).
 # "sweep" is the mean over one pass of the 14 shapes; algorithmic bytes are 226.5 MB resp. 335.5 MB.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"sweep": 536.6e6, "M10": 939.9e6}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"sweep": 544.9e6, "M10": 939.8e6}
 RAMP_MS = 40.0       # continuous load queued ahead of every timed region (engine-clock ramp)
 
 
