@@ -31,12 +31,12 @@ class RocBLAS:
     (the kernel library for the GPU is read lazily); both happen outside any timed region."""
 
     def __init__(self, library: Optional[str] = None):
-        hip.init()
         path = library or str(Path(hip.ROCM) / "lib" / "librocblas.so")
         try:
             self._lib = C.CDLL(path)
         except OSError as e:
             raise VendorBlasError(f"cannot load rocBLAS ({path}): {e}") from e
+        hip.init()
         L = self._lib
         L.rocblas_create_handle.argtypes = [C.POINTER(C.c_void_p)]
         L.rocblas_destroy_handle.argtypes = [C.c_void_p]

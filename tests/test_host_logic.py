@@ -202,3 +202,9 @@ def test_plot_results_writes_an_image(tmp_path):
     df = pd.DataFrame({"Roller TFLOPS": [139.0, 148.5, 120.0], "Speedup vs Host": [37.0, 40.2, 0]})
     out = bm.plot_results(df, tmp_path / "sweep.png")
     assert out.exists() and out.stat().st_size > 5000 and out.read_bytes()[:4] == b"\x89PNG"
+
+
+def test_vendor_library_missing_is_reported_not_fatal(tmp_path):
+    from mlir_roller_amd.vendor_blas import RocBLAS, VendorBlasError
+    with pytest.raises(VendorBlasError, match="cannot load rocBLAS"):
+        RocBLAS(library=str(tmp_path / "librocblas.so"))
