@@ -248,6 +248,8 @@ class Policy:
     # registers per lane the MFMA kernel needs besides its accumulators and operand fragments:
     # addresses, loop state, buffer resources (measured: 40-60)
     REG_OVERHEAD = 50
+    # wave tiles of at most this many elements list the 16x16x4 variant first
+    SMALL_WAVE_TILE = 64 * 64
 
     def __init__(self, config: MatmulConfig, arch: TileDevice) -> None:
         self.arch = arch
@@ -462,6 +464,12 @@ class Policy:
             td.mfma = mi
             td.threads = block_size
             out.append(td.clone())
+        # The instruction with the longer k (16x16x4) moves half as many accumulator bytes per FLOP,
+        # which leaves the register file free for LDS fragment reads: it wins on small wave tiles,
+        # where those reads are dense (measured 1-2 % on wave tiles up to 64x64); the larger
+        # instruction wins on large ones.
+        if len(out) > 1 and math.prod(out[0].wave_tile) <= self.SMALL_WAVE_TILE:
+            out.sort(key=lambda t: t.mfma)
         return out
 
     # ---- top level ------------------------------------------------------------------------------

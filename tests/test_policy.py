@@ -342,3 +342,12 @@ def test_mi355x_top_hints_compile_without_spills_or_scratch():
         res = hip.code_object_resources(hip.compile_config(g))
         assert res["vgpr_spills"] == 0 and res["sgpr_spills"] == 0 and res["scratch_bytes"] == 0, (shape, g.tag(), res)
         assert 0 < res["vgprs"] <= 512 // max(1, g.threads // 256), (g.tag(), res)
+
+
+def test_mi355x_small_wave_tiles_list_the_long_k_instruction_first():
+    arch = MI355X()
+    first = lambda shape: get_roller_hints(MatmulConfig(*shape, 32), arch, topk=2)
+    a, b = first((2048, 2048, 2048))                       # 128x128 over eight waves: 32x64 wave tiles
+    assert (a.wave_tile, a.mfma, b.wave_tile, b.mfma) == ([32, 64], 16, [32, 64], 32)
+    a, b = first((4096, 8192, 4096))                       # 64x128 and larger: 32x32x2 first
+    assert a.mfma == 32 and b.mfma == 32 and a.wave_tile == [64, 128]
