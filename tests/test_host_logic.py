@@ -9,7 +9,6 @@ from mlir_roller_amd import benchmark as bm
 from mlir_roller_amd import roller
 from mlir_roller_amd.analyze import MatmulConfig, get_roller_hints
 from mlir_roller_amd.arch import CUDA, MI355X
-from mlir_roller_amd.hip import GemmConfig
 
 
 def test_hint_to_gemm_config_aligned_problem():
