@@ -18,7 +18,8 @@ The line also carries
                 taken on the stream the kernels run on;
   cpu_baseline  numpy float32 matmul (its BLAS, all host cores) timed on the same inputs, one
                 pass over the workload; a reported figure, not a target;
-  per_shape     ms, TFLOP/s, % of peak, winning hint and its rank for every shape.
+  per_shape     ms (mean of a batch, minimum and median of single launches), TFLOP/s, % of peak,
+                winning hint and its rank for every shape.
 """
 
 from __future__ import annotations
@@ -307,8 +308,17 @@ def main() -> int:
     for c in cases:
         M, N, K = c["shape"]
         ms = time_plan(c["plan"], c["bufs"], c["shape"], reps=max(args.steps, 5), warm=2)
+        # spread of single launches: an event after every launch of a second batch that follows at once
+        marks = [Event() for _ in range(max(args.steps, 5) + 1)]
+        marks[0].record(stream)
+        for mark in marks[1:]:
+            c["plan"].launch(c["bufs"][0], c["bufs"][1], c["bufs"][2], M, N, K, stream=stream)
+            mark.record(stream)
+        marks[-1].synchronize()
+        each = sorted(hip.get_elapsed_time(a, b) for a, b in zip(marks, marks[1:]))
         tf = 2.0 * M * N * K / ms / 1e9
-        per_shape.append({"name": c["name"], "M": M, "N": N, "K": K, "ms": round(ms, 5), "tflops": round(tf, 2),
+        per_shape.append({"name": c["name"], "M": M, "N": N, "K": K, "ms": round(ms, 5),
+                          "min_ms": round(each[0], 5), "median_ms": round(each[len(each) // 2], 5), "tflops": round(tf, 2),
                           "pct_of_peak": round(100 * tf / PEAK_TFLOPS, 1), "kernel": c["cfg"].tag(),
                           "hint_rank": c["rank"], "hints": c["hints"], "top1_over_best": c["top1_over_best"],
                           "normwise_err": c["rep"]["normwise"], "max_abs_err": c["rep"]["max_abs"],
