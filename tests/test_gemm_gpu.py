@@ -133,6 +133,24 @@ def test_matches_oracle_within_tolerance_and_exactly_on_integers(device, cfg, sh
     assert np.array_equal(run_gemm(cfg, Ai, Bi), go.c_gemm_f32(Ai, Bi))
 
 
+def test_committed_exact_cases_on_the_gpu(device):
+    """The committed integer known answers (tests/golden/gemm_exact_cases.json), bit for bit, through a dword
+    kernel, a 128-bit kernel where the shape allows it, the direct-to-LDS kernel and the transposed-operand kernel."""
+    import json
+    from pathlib import Path
+    cases = json.loads((Path(__file__).resolve().parent / "golden" / "gemm_exact_cases.json").read_text())
+    for case in cases:
+        A, B = np.array(case["A"], np.float32), np.array(case["B"], np.float32)
+        want = np.array(case["C"], np.float32)
+        cfgs = [GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 1, 1), GemmConfig(64, 64, 16, 16, 64, 16, 3, 4, 4, 1, 1, 3, 8, 0, 0, 1)]
+        if case["K"] % 4 == 0 and case["N"] % 4 == 0:
+            cfgs += [GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1), GemmConfig(128, 128, 32, 32, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1),
+                     GemmConfig(128, 128, 32, 32, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1)]
+        for cfg in cfgs:
+            say("golden", case["name"], cfg.tag())
+            assert np.array_equal(run_gemm(cfg, A, B), want), (case["name"], cfg.tag())
+
+
 def test_structured_operands_are_exact(device):
     cfg = GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1)
     n = 200

@@ -131,3 +131,21 @@ def test_make_inputs_is_seeded_and_in_range():
     assert set(np.unique(Ai)).issubset(set(range(10)))
     An, _ = go.make_inputs(200, 9, 200, seed=3, distribution="normal")
     assert abs(float(An.mean())) < 0.05 and abs(float(An.std()) - 1) < 0.05
+
+
+def golden_cases():
+    import json
+    from pathlib import Path
+    return json.loads((Path(__file__).resolve().parent / "golden" / "gemm_exact_cases.json").read_text())
+
+
+@pytest.mark.parametrize("case", golden_cases(), ids=lambda c: c["name"])
+def test_committed_exact_cases(case):
+    """Known answers computed with Python integers (tests/golden/make_gemm_golden.py): every routine of the
+    oracle reproduces them bit for bit, also through a transposed copy of B."""
+    A, B = np.array(case["A"], np.float32), np.array(case["B"], np.float32)
+    C = np.array(case["C"], np.float64)
+    assert A.shape == (case["M"], case["K"]) and B.shape == (case["K"], case["N"]) and C.shape == (case["M"], case["N"])
+    for routine in (go.gemm_f32, go.gemm_f64, go.c_gemm_f32, go.c_gemm_f64, go.c_gemm_naive):
+        assert np.array_equal(np.asarray(routine(A, B), dtype=np.float64), C), routine.__name__
+    assert np.array_equal(np.array(go.gemm_exact(A, B), dtype=np.float64), C)
