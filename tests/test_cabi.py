@@ -157,3 +157,38 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     with pytest.raises(HipError) as err:
         hip.lib()
     assert "missing" in str(err.value)
+
+
+def test_concurrent_precompiles_and_thread_local_errors(hip_lib, tmp_path):
+    """ctypes releases the GIL inside the library: eight threads compile into one cache directory and
+    provoke errors at the same time; every thread sees its own error text and every entry is intact."""
+    import threading
+    results, errors = {}, {}
+
+    def work(i):
+        try:
+            cfg = GemmConfig(64, 64, 16, 32, 32, 32, 1 + i % 3, 4, 0, 4, i % 2)
+            results[i] = hip.precompile(cfg)
+            try:
+                hip.config_check(GemmConfig(64, 64, 16, 32, 32, 32, 2, 4, 0, 4 + i, 0))     # vec = 4 + i is invalid
+            except HipError as e:
+                errors[i] = str(e)
+        except Exception as e:                                                              # pragma: no cover
+            errors[i] = f"unexpected: {e!r}"
+
+    try:
+        hip.set_cache_dir(tmp_path)
+        threads = [threading.Thread(target=work, args=(i,)) for i in range(1, 9)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join(timeout=120)
+        assert sorted(results) == list(range(1, 9)) and all(v > 1000 for v in results.values())
+        for i in range(1, 9):
+            assert f"got {4 + i}" in errors[i], errors[i]                                   # its own message, not a neighbour's
+        files = list(tmp_path.glob("gemm_*.hsaco"))
+        assert len(files) == 6 and not list(tmp_path.glob("*.tmp*"))                          # 3 depths x 2 edge modes
+        for f in files:
+            assert f.read_bytes()[:4] == b"\x7fELF" and f.read_bytes()[-16:-12] == b"RLHC"
+    finally:
+        hip.set_cache_dir(hip.DEFAULT_CACHE_DIR)
