@@ -4,6 +4,11 @@ that the build step can compile the same kernel configurations ahead of time."""
 
 import numpy as np
 
+# vectors, slivers and a very long K, as (M, N, K)
+EXTREME_SHAPES = [(1, 1, 1), (1, 7, 3), (100000, 8, 64), (8, 100000, 64), (64, 64, 100000), (65536, 128, 128),
+                  (3, 50000, 5), (50000, 3, 5), (257, 255, 1023), (4096, 4, 4096), (4, 4096, 4096), (1, 4096, 4096),
+                  (4096, 1, 4096)]
+
 
 def seeded_policy_cases(arch, count: int = 40, seed: int = 20240607):
     """Yields ``(case, matmul_config, hint, depth, trans_b, accumulate)``; ragged and tiny

@@ -490,6 +490,26 @@ def test_vendor_baseline_is_a_correct_row_major_gemm(device):
     assert ms > 0 and gflops == pytest.approx(2 * 512 * 768 * 256 * 1e-9 / (ms / 1e3), rel=1e-6)
 
 
+from gemm_cases import EXTREME_SHAPES  # noqa: E402  (beside this file; the build step compiles the same kernels ahead)
+
+
+@pytest.mark.parametrize("shape", EXTREME_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_extreme_aspect_ratios_through_policy(device, shape):
+    """Vectors, slivers and a very long K: the policy's first hint compiles, launches and is exact
+    (entries in {-2..2}, so sums stay below 2^24 even for K = 100000)."""
+    M, N, K = shape
+    mc = MatmulConfig(M, N, K, 32)
+    hint = get_roller_hints(mc, MI355X(), topk=1)[0]
+    func = roller.Compiler(mc, hint, bm.PIPELINE_DEPTH).compile()
+    say("extreme", shape, func.gemm_config.tag())
+    A, B = small_integer_matrix(M, K, 3), small_integer_matrix(K, N, 4)
+    dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray((M, N))
+    dC.fill_bytes(0xFF)
+    func(func.grid_dims(), func.block_dims(), (dA, dB, dC))
+    hip.synchronize()
+    assert np.array_equal(dC.get(), A @ B)
+
+
 def test_handle_checks_grid_and_block(device):
     cfg = MatmulConfig(512, 512, 128, 32)
     hint = get_roller_hints(cfg, MI355X(), topk=1)[0]
