@@ -91,3 +91,39 @@ def test_transposed_operand_rows_are_a_permutation_that_matches_the_epilogue(wn,
     # column w*wn + (bj // vn)*mi*vn + vn*lane + bj % vn
     for w, bj, lane in itertools.product(range(waves_n), range(tn), range(mi)):
         assert col_of_row(w * wn + bj * mi + lane) == w * wn + (bj // vn) * mi * vn + vn * lane + bj % vn
+
+
+@pytest.mark.parametrize("wn,mi", [(32, 32), (64, 32), (128, 32), (256, 32), (16, 16), (32, 16), (64, 16), (128, 16)])
+def test_column_interleave_covers_every_column_once_and_matches_the_epilogue(wn, mi):
+    """B[K, N] operand: a lane reads VN consecutive columns at wn0 + v*MI*VN + VN*lane and element e of that
+    read feeds block v*VN + e; the epilogue stores block bj's accumulator to column (bj//VN)*MI*VN + VN*lane + bj%VN."""
+    assert "wn0 + VN * lr;  // + (kk+t)*LDB_S + v*MI*VN" in TEMPLATE and "const int col = wn0 + v * MI * VN + VN * lr;" in TEMPLATE
+    tn = wn // mi
+    vn = 4 if tn >= 4 else tn
+    nvb = tn // vn
+    fed = {}                                        # (block, lane) -> column whose B values the block's MFMA receives
+    for v, lane, e in itertools.product(range(nvb), range(mi), range(vn)):
+        fed[(v * vn + e, lane)] = v * mi * vn + vn * lane + e
+    assert sorted(fed.values()) == list(range(wn))                  # the wave tile's columns, each exactly once
+    for (bj, lane), col in fed.items():
+        assert col == (bj // vn) * mi * vn + vn * lane + bj % vn    # where the epilogue writes that accumulator
+    # a lane's VN stores are adjacent, so they leave as one vector store
+    for v, lane in itertools.product(range(nvb), range(mi)):
+        cols = [fed[(v * vn + e, lane)] for e in range(vn)]
+        assert cols == list(range(cols[0], cols[0] + vn)) and cols[0] % vn == 0
+
+
+@pytest.mark.parametrize("mi", [32, 16])
+def test_k_permutation_pairs_the_same_k_on_both_operands(mi):
+    """MFMA t of a round contracts k = kk + 4*g + t for lane group g: A takes element t of the 128-bit read at
+    k offset 4*g, B is read from row kk + 4*g + t; over the 4 MFMAs and 64/mi groups every k of the round once."""
+    assert "const int b_frag = (4 * lg) * LDB_S + wn0 + VN * lr;" in TEMPLATE and "f.b[t][v] = *(const bvec_t*)&Bs[b_frag + (kk + t) * LDB_S" in TEMPLATE
+    kg = 64 // mi
+    ksuper = 4 * kg
+    seen = []
+    for t, g in itertools.product(range(4), range(kg)):
+        a_k = 4 * g + t                  # element t of the A read that starts at k offset 4*g
+        b_row = 4 * g + t                # b_frag's row offset 4*g plus (kk + t)
+        assert a_k == b_row
+        seen.append(a_k)
+    assert sorted(seen) == list(range(ksuper))
