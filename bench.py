@@ -232,8 +232,31 @@ def main() -> int:
             hip.synchronize()
             for (rank, g, text, plan), (e0, e1) in zip(plans, marks):
                 ranked.append((hip.get_elapsed_time(e0, e1) / 10, rank, g, text))
-            tune_s += time.perf_counter() - t0
             ranked.sort(key=lambda r: r[0])
+            # Near ties are common (several hints within 0.5 %): the four fastest are timed again,
+            # longer and twice in alternation, and ordered by the better of their two means.
+            finalists = ranked[:4]
+            if len(finalists) > 1:
+                by_rank = {rank: plan for rank, _, _, plan in plans}
+                time_plan(by_rank[finalists[0][1]], bufs, shape, reps=1, warm=0)
+                marks = []
+                for _ in range(2):
+                    for _, rank, _, _ in finalists:
+                        for _ in range(2):
+                            by_rank[rank].launch(bufs[0], bufs[1], bufs[2], M, N, K, stream=stream)
+                        e0, e1 = Event(), Event()
+                        e0.record(stream)
+                        for _ in range(30):
+                            by_rank[rank].launch(bufs[0], bufs[1], bufs[2], M, N, K, stream=stream)
+                        e1.record(stream)
+                        marks.append((rank, e0, e1))
+                hip.synchronize()
+                again = {}
+                for rank, e0, e1 in marks:
+                    again[rank] = min(again.get(rank, float("inf")), hip.get_elapsed_time(e0, e1) / 30)
+                finalists = sorted(((again[rank], rank, g, text) for _, rank, g, text in finalists), key=lambda r: r[0])
+                ranked = finalists + ranked[4:]
+            tune_s += time.perf_counter() - t0
         if not ranked:
             log(f"[bench] {name}: no usable hint")
             return 1
