@@ -13,8 +13,11 @@
  *   - one device per process (the reference pins one GPU through its environment, .env:5-6);
  *     calls are synchronous with respect to the host except rl_launch / rl_gemm_* / rl_event_record,
  *     which enqueue on the given stream (NULL = the default stream).
- *   - the library is thread-safe for concurrent calls that use different plans/modules; error
- *     text is thread-local.
+ *   - the library is thread-safe: every entry point selects the device of rl_init on the calling
+ *     thread, plan creation and the cache directory are serialised, launches of plans may run
+ *     concurrently with each other, and rl_gemm_plans_clear waits for running launch calls and for
+ *     the device before it unloads anything.  rl_module_unload likewise drains the device first.
+ *     Error text is thread-local.
  */
 #ifndef ROLLER_HIP_H
 #define ROLLER_HIP_H
@@ -104,6 +107,9 @@ void rl_free_host(void* p);
 int rl_module_load(const void* code, rl_module* out);
 int rl_module_get_function(rl_module m, const char* name, rl_function* out);
 int rl_module_unload(rl_module m);
+/* Fails with RL_ERR_INVALID_ARG and text when the runtime grants less than `bytes` (the limit is
+ * read back after the opt-in: function attribute where the runtime keeps one, otherwise the
+ * device's per-workgroup LDS minus the function's static LDS). */
 int rl_func_set_max_dynamic_lds(rl_function f, int bytes);
 
 /* Launches f.  `args` holds n_args pointers, one per kernel parameter, each pointing at that
@@ -160,6 +166,10 @@ int rl_gemm_precompile(const rl_gemm_config* cfg, size_t* code_size);
 int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* compile_ms);
 int rl_gemm_plan_function(const rl_gemm_plan* plan, rl_function* out);
 int rl_gemm_plan_lds_bytes(const rl_gemm_plan* plan);
+/* Dynamic LDS bytes the runtime grants the plan's kernel, read back after the opt-in that the
+ * reference does with funcSetAttribute(MAX_DYNAMIC_SHARED_SIZE_BYTES) (src/roller.py:508-510);
+ * rl_gemm_plan_create fails with text when it is below rl_gemm_plan_lds_bytes. */
+int rl_gemm_plan_lds_limit(const rl_gemm_plan* plan);
 int rl_gemm_plan_threads(const rl_gemm_plan* plan);
 /* Kernel resource usage read from the code object's metadata (-1 if unknown). */
 int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int* sgprs,

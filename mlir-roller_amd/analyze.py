@@ -94,6 +94,23 @@ def compute_memory_traffic(output_tile: List[int], matmul_config: MatmulConfig, 
     return moved * eb
 
 
+# Pipeline depth the MI355X sweep runs at (the reference's sweep runs its depth 2,
+# /root/reference/src/benchmark.py:29): two LDS buffers plus a register stage.
+DEFAULT_PIPELINE_DEPTH = 3
+
+
+def loads_go_direct_to_lds(matmul_config: "MatmulConfig", block_tile: Sequence[int], rstep: int,
+                           pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> bool:
+    """Whether the MFMA kernel built for this tile uses its direct-to-LDS path (unpadded,
+    XOR-swizzled rows; no staging registers): only at pipeline depth 3, with 128-bit global
+    accesses (K and N multiples of 4), a power-of-two reduce step, and operand tiles that are
+    whole waves of 16-byte units.  The policy's LDS and register models and the mapping from a
+    hint to template parameters all ask this one function."""
+    m, n = block_tile
+    return (pipeline_depth >= 3 and matmul_config.K % 4 == 0 and matmul_config.N % 4 == 0
+            and rstep & (rstep - 1) == 0 and (m * rstep // 4) % 64 == 0 and (rstep * n // 4) % 64 == 0)
+
+
 def _natural_size(nbytes: float) -> str:
     """1536 -> '1.5 KiB' (binary units, one decimal)."""
     if abs(nbytes) < 1024:
@@ -121,6 +138,7 @@ class TileDict:
         self.mfma = 0
         self.threads = 0
         self.lds_row_pad = 0
+        self.pipeline_depth = DEFAULT_PIPELINE_DEPTH
         # analysis
         self.traffic = -1
         self.smem_cost = -1
@@ -156,19 +174,22 @@ class TileDict:
         """Bytes of workgroup memory for one pipeline stage: an [m, rstep] and an [rstep, n] tile."""
         step = self.rstep if rstep is None else rstep
         cfg = self.matmul_config
-        # The MFMA kernel keeps the [m, rstep] tile unpadded only on its direct-to-LDS path: K and N
-        # multiples of 4 and a power-of-two step.  Otherwise every row grows by ``lds_row_pad``.
-        swizzled = cfg.K % 4 == 0 and cfg.N % 4 == 0 and step & (step - 1) == 0
-        pad = 0 if swizzled else self.lds_row_pad
+        # The MFMA kernel keeps the [m, rstep] tile unpadded only on its direct-to-LDS path;
+        # otherwise every row grows by ``lds_row_pad`` wherever that keeps its 128-bit reads
+        # conflict-free (an even number of 16-byte units per row).
+        pad = self.lds_row_pad
+        if not pad or (step // 4) % 2 or loads_go_direct_to_lds(cfg, self.block_tile, step, self.pipeline_depth):
+            pad = 0
         return (step * sum(self.block_tile) + pad * self.block_tile[0]) * cfg.el_bytes
 
     @classmethod
     def from_block_tile(cls, block_tile: List[int], rstep: int, matmul_config: MatmulConfig,
-                        arch: TileDevice) -> "TileDict":
+                        arch: TileDevice, pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> "TileDict":
         """Cost model of one block tile.  A tile that overflows workgroup memory or the register
         file comes back with ``valid = False`` and its analysis fields still at -1."""
         td = cls(block_tile, matmul_config, rstep)
         td.lds_row_pad = arch.lds_row_pad
+        td.pipeline_depth = pipeline_depth
 
         td.smem_cost = td.infer_smem_usage()
         if td.smem_cost > arch.smem_cap:
@@ -251,9 +272,13 @@ class Policy:
     # wave tiles of at most this many elements list the 16x16x4 variant first
     SMALL_WAVE_TILE = 64 * 64
 
-    def __init__(self, config: MatmulConfig, arch: TileDevice) -> None:
+    def __init__(self, config: MatmulConfig, arch: TileDevice,
+                 pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> None:
         self.arch = arch
         self.matmul_config = config
+        # depth the kernels will be built at: decides whether the LDS tiles are padded and
+        # whether loads are staged through registers (both cost model inputs on MI355X)
+        self.pipeline_depth = pipeline_depth
 
     # ---- device-model helpers -------------------------------------------------------------
 
@@ -347,7 +372,7 @@ class Policy:
 
         tiles = []
         for m, n in itertools.product(*steps):
-            td = TileDict.from_block_tile([m, n], rstep, self.matmul_config, self.arch)
+            td = TileDict.from_block_tile([m, n], rstep, self.matmul_config, self.arch, self.pipeline_depth)
             if td.valid:
                 tiles.append(td)
         return sorted(tiles, key=self._priority)
@@ -426,9 +451,7 @@ class Policy:
         it also stages one K step of both operand tiles in registers."""
         blocks_m, blocks_n = wave_tile[0] // mi, wave_tile[1] // mi
         regs = self.REG_OVERHEAD + 2 * 4 * (blocks_m + blocks_n)
-        cfg = self.matmul_config
-        direct = cfg.K % 4 == 0 and cfg.N % 4 == 0 and td.rstep & (td.rstep - 1) == 0
-        if not direct:
+        if not loads_go_direct_to_lds(self.matmul_config, td.block_tile, td.rstep, self.pipeline_depth):
             regs += -(-(sum(td.block_tile) * td.rstep) // block_size)
         return regs
 
@@ -486,6 +509,9 @@ class Policy:
         return hints
 
 
-def get_roller_hints(matmul_config: MatmulConfig, arch: TileDevice, topk: int = 10) -> List[TileDict]:
-    """Top-``topk`` tile configurations for ``matmul_config`` on ``arch``, best first."""
-    return Policy(matmul_config, arch).emit_config(topk)
+def get_roller_hints(matmul_config: MatmulConfig, arch: TileDevice, topk: int = 10,
+                     pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> List[TileDict]:
+    """Top-``topk`` tile configurations for ``matmul_config`` on ``arch``, best first.
+    ``pipeline_depth`` (not in the reference's signature) is the depth the kernels will be
+    compiled at; it only matters on device models with matrix cores."""
+    return Policy(matmul_config, arch, pipeline_depth).emit_config(topk)

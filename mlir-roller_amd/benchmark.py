@@ -24,11 +24,11 @@ from typing import List, Optional, Sequence, Tuple
 
 import pandas as pd
 
-from .analyze import MatmulConfig, get_roller_hints
+from .analyze import DEFAULT_PIPELINE_DEPTH, MatmulConfig, get_roller_hints
 from .arch import MI355X, TileDevice
 from .roller import Compiler, run_baseline, run_eval, run_vendor_baseline
 
-PIPELINE_DEPTH = 3
+PIPELINE_DEPTH = DEFAULT_PIPELINE_DEPTH
 
 # The fourteen shapes of the reference's result table, M0..M13 as (M, N, K) (README.md:13-17).
 README_SHAPES: List[Tuple[int, int, int]] = [
@@ -82,7 +82,7 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
         print(f"Generating and testing {topk} roller hints...")
         t0 = time.perf_counter()
         try:
-            hints = get_roller_hints(config, arch, topk=topk)
+            hints = get_roller_hints(config, arch, topk=topk, pipeline_depth=pipeline_depth)
         except Exception as e:
             print(f"Could not get hints for shape ({m},{n},{k}): {e}")
             hints = []

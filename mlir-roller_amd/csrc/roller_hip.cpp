@@ -22,6 +22,7 @@
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <shared_mutex>
 #include <string>
 #include <vector>
 
@@ -64,8 +65,12 @@ int hip_fail(hipError_t e, const char* what) {
   } while (0)
 
 std::mutex g_mutex;  // guards the cache directory, the plan table and initialisation
+// Launches of a plan hold this shared; rl_gemm_plans_clear holds it exclusively while it unloads
+// the modules, so a launch never reads a function handle that is being torn down.
+std::shared_mutex g_plans_rw;
 std::atomic<bool> g_ready{false};  // read without the lock on every entry point
 std::atomic<int> g_device{-1};
+std::atomic<int> g_lds_limit{0};   // largest LDS allocation of one workgroup, read from the device at rl_init
 std::string g_cache_dir;
 
 struct Plan {
@@ -73,6 +78,7 @@ struct Plan {
   hipModule_t module = nullptr;
   hipFunction_t func = nullptr;
   int lds_bytes = 0;
+  int lds_limit = 0;  // dynamic LDS the runtime grants this function, read back after load
   int threads = 0;
   int vgprs = -1, agprs = -1, sgprs = -1, spilled = -1, scratch = -1;
 };
@@ -302,25 +308,56 @@ int metadata_int(const std::vector<char>& code, const char* key) {
   return -1;
 }
 
-// Workgroups that want more than 64 KB of dynamic LDS opt in per function.  The runtime keys this
-// attribute by host-side kernel stubs; for a function that came from hipModuleGetFunction it may
-// answer "invalid device function", which means that no opt-in exists for module functions and
-// the launch itself is the check.  Only that answer is tolerated.
-int opt_in_lds(hipFunction_t f, int bytes) {
-  hipError_t e = hipFuncSetAttribute((const void*)f, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (e == hipSuccess) return RL_OK;
-  if (e == hipErrorInvalidDeviceFunction) {
-    (void)hipGetLastError();  // do not leave a sticky error for the next call
-    return RL_OK;
-  }
-  return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
-}
-
 // The current device is a per-thread setting of the HIP runtime; a thread other than the one that
-// called rl_init would otherwise work on device 0.
+// called rl_init would otherwise work on device 0.  Every entry point that reaches the runtime
+// goes through here; the device is set once per thread.
 int ensure_ready() {
   if (!g_ready) return fail(RL_ERR_NO_DEVICE, "rl_init has not been called (or failed)");
-  HIP_TRY(hipSetDevice(g_device));
+  thread_local int t_device = -1;
+  if (t_device != g_device) {
+    HIP_TRY(hipSetDevice(g_device));
+    t_device = g_device;
+  }
+  return RL_OK;
+}
+
+#define READY_OR_RETURN()      \
+  do {                         \
+    int rc_ = ensure_ready();  \
+    if (rc_) return rc_;       \
+  } while (0)
+
+// Workgroups that want more than 64 KB of dynamic LDS opt in per function, and the answer is read
+// back: *granted receives the dynamic LDS size the runtime will accept for f.  The runtime keys the
+// opt-in attribute by host-side kernel stubs; for a function that came from hipModuleGetFunction it
+// may answer "invalid device function" (no opt-in exists for module functions).  Only that answer
+// is tolerated, and then -- as whenever the function attribute cannot be read -- the grant is the
+// device's per-workgroup LDS limit minus the function's static LDS.
+int opt_in_lds(hipFunction_t f, int bytes, int* granted) {
+  if (bytes > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)f, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipErrorInvalidDeviceFunction) {
+      (void)hipGetLastError();  // do not leave a sticky error for the next call
+    } else if (e != hipSuccess) {
+      return hip_fail(e, "hipFuncSetAttribute(MaxDynamicSharedMemorySize)");
+    }
+  }
+  int static_lds = 0, dynamic_max = 0;
+  if (hipFuncGetAttribute(&static_lds, HIP_FUNC_ATTRIBUTE_SHARED_SIZE_BYTES, f) != hipSuccess) {
+    (void)hipGetLastError();
+    static_lds = 0;
+  }
+  if (hipFuncGetAttribute(&dynamic_max, HIP_FUNC_ATTRIBUTE_MAX_DYNAMIC_SHARED_SIZE_BYTES, f) != hipSuccess) {
+    (void)hipGetLastError();
+    dynamic_max = 0;
+  }
+  const int device_room = g_lds_limit.load() - static_lds;
+  // A function attribute of 0 means "never set": the device limit applies.
+  const int limit = dynamic_max > 0 ? (dynamic_max < device_room ? dynamic_max : device_room) : device_room;
+  if (granted) *granted = limit;
+  if (bytes > limit)
+    return fail(RL_ERR_INVALID_ARG, "kernel needs %d bytes of dynamic LDS, the runtime grants %d (device limit %d, static %d, function attribute %d)",
+                bytes, limit, g_lds_limit.load(), static_lds, dynamic_max);
   return RL_OK;
 }
 
@@ -345,6 +382,11 @@ int rl_init(int device) {
   HIP_TRY(hipGetDeviceProperties(&prop, device));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
     return fail(RL_ERR_NO_DEVICE, "device %d is %s; this library is built for gfx950 (MI355X) only", device, prop.gcnArchName);
+  int lds_limit = (int)prop.sharedMemPerBlockOptin > 0 ? (int)prop.sharedMemPerBlockOptin : (int)prop.sharedMemPerBlock;
+  int attr = 0;
+  if (hipDeviceGetAttribute(&attr, hipDeviceAttributeMaxSharedMemoryPerBlock, device) == hipSuccess && attr > lds_limit)
+    lds_limit = attr;
+  g_lds_limit = lds_limit;
   g_device = device;
   g_ready = true;
   return RL_OK;
@@ -361,7 +403,7 @@ int rl_device_info(rl_device_props* out) {
   snprintf(out->arch, sizeof out->arch, "%.63s", p.gcnArchName);
   out->compute_units = p.multiProcessorCount;
   out->wavefront_size = p.warpSize;
-  out->lds_bytes_per_block = (int)p.sharedMemPerBlockOptin > 0 ? (int)p.sharedMemPerBlockOptin : (int)p.sharedMemPerBlock;
+  out->lds_bytes_per_block = g_lds_limit.load();
   out->regs_per_block = p.regsPerBlock;
   out->l2_bytes = p.l2CacheSize;
   out->clock_khz = p.clockRate;
@@ -411,6 +453,7 @@ int rl_module_load(const void* code, rl_module* out) {
 
 int rl_module_get_function(rl_module m, const char* name, rl_function* out) {
   if (!m || !name || !out) return fail(RL_ERR_INVALID_ARG, "rl_module_get_function: NULL argument");
+  READY_OR_RETURN();
   hipFunction_t f = nullptr;
   HIP_TRY(hipModuleGetFunction(&f, (hipModule_t)m, name));
   *out = f;
@@ -419,6 +462,10 @@ int rl_module_get_function(rl_module m, const char* name, rl_function* out) {
 
 int rl_module_unload(rl_module m) {
   if (!m) return RL_OK;
+  READY_OR_RETURN();
+  // kernels of this module may still be queued (a host wrapper's destructor can get here right
+  // after its last launch): let them finish before their code goes away
+  HIP_TRY(hipDeviceSynchronize());
   HIP_TRY(hipModuleUnload((hipModule_t)m));
   return RL_OK;
 }
@@ -426,7 +473,8 @@ int rl_module_unload(rl_module m) {
 int rl_func_set_max_dynamic_lds(rl_function f, int bytes) {
   if (!f || bytes < 0) return fail(RL_ERR_INVALID_ARG, "rl_func_set_max_dynamic_lds: bad argument");
   if (bytes > 160 * 1024) return fail(RL_ERR_INVALID_ARG, "%d bytes of LDS exceed the 160 KB of a CU", bytes);
-  return opt_in_lds((hipFunction_t)f, bytes);
+  READY_OR_RETURN();
+  return opt_in_lds((hipFunction_t)f, bytes, nullptr);
 }
 
 int rl_launch(rl_function f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by,
@@ -436,6 +484,9 @@ int rl_launch(rl_function f, unsigned gx, unsigned gy, unsigned gz, unsigned bx,
   if ((unsigned long)bx * by * bz > 1024) return fail(RL_ERR_INVALID_ARG, "rl_launch: more than 1024 threads per block");
   for (int i = 0; i < n_args; ++i)
     if (!args[i]) return fail(RL_ERR_INVALID_ARG, "rl_launch: args[%d] is NULL", i);
+  if ((long)lds_bytes > g_lds_limit.load() && g_ready)
+    return fail(RL_ERR_INVALID_ARG, "rl_launch: %u bytes of dynamic LDS exceed the device's %d per workgroup", lds_bytes, g_lds_limit.load());
+  READY_OR_RETURN();
   HIP_TRY(hipModuleLaunchKernel((hipFunction_t)f, gx, gy, gz, bx, by, bz, lds_bytes, (hipStream_t)stream, args, nullptr));
   return RL_OK;
 }
@@ -452,6 +503,7 @@ int rl_malloc(void** dptr, size_t bytes) {
 
 int rl_free(void* dptr) {
   if (!dptr) return RL_OK;
+  READY_OR_RETURN();
   HIP_TRY(hipFree(dptr));
   return RL_OK;
 }
@@ -459,6 +511,7 @@ int rl_free(void* dptr) {
 int rl_memcpy_h2d(void* dst, const void* src, size_t bytes) {
   if (bytes == 0) return RL_OK;
   if (!dst || !src) return fail(RL_ERR_INVALID_ARG, "rl_memcpy_h2d: NULL argument");
+  READY_OR_RETURN();
   HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
   return RL_OK;
 }
@@ -466,6 +519,7 @@ int rl_memcpy_h2d(void* dst, const void* src, size_t bytes) {
 int rl_memcpy_d2h(void* dst, const void* src, size_t bytes) {
   if (bytes == 0) return RL_OK;
   if (!dst || !src) return fail(RL_ERR_INVALID_ARG, "rl_memcpy_d2h: NULL argument");
+  READY_OR_RETURN();
   HIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
   return RL_OK;
 }
@@ -473,6 +527,7 @@ int rl_memcpy_d2h(void* dst, const void* src, size_t bytes) {
 int rl_memset(void* dptr, int byte_value, size_t bytes) {
   if (bytes == 0) return RL_OK;
   if (!dptr) return fail(RL_ERR_INVALID_ARG, "rl_memset: NULL argument");
+  READY_OR_RETURN();
   HIP_TRY(hipMemset(dptr, byte_value, bytes));
   return RL_OK;
 }
@@ -489,6 +544,7 @@ int rl_stream_create(rl_stream* out) {
 
 int rl_stream_destroy(rl_stream s) {
   if (!s) return RL_OK;
+  READY_OR_RETURN();
   HIP_TRY(hipStreamDestroy((hipStream_t)s));
   return RL_OK;
 }
@@ -505,24 +561,28 @@ int rl_event_create(rl_event* out) {
 
 int rl_event_record(rl_event e, rl_stream s) {
   if (!e) return fail(RL_ERR_INVALID_ARG, "rl_event_record: NULL event");
+  READY_OR_RETURN();
   HIP_TRY(hipEventRecord((hipEvent_t)e, (hipStream_t)s));
   return RL_OK;
 }
 
 int rl_event_sync(rl_event e) {
   if (!e) return fail(RL_ERR_INVALID_ARG, "rl_event_sync: NULL event");
+  READY_OR_RETURN();
   HIP_TRY(hipEventSynchronize((hipEvent_t)e));
   return RL_OK;
 }
 
 int rl_event_elapsed_ms(rl_event start, rl_event stop, float* ms) {
   if (!start || !stop || !ms) return fail(RL_ERR_INVALID_ARG, "rl_event_elapsed_ms: NULL argument");
+  READY_OR_RETURN();
   HIP_TRY(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
   return RL_OK;
 }
 
 int rl_event_destroy(rl_event e) {
   if (!e) return RL_OK;
+  READY_OR_RETURN();
   HIP_TRY(hipEventDestroy((hipEvent_t)e));
   return RL_OK;
 }
@@ -616,11 +676,18 @@ int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* co
       return rc;
     }
   }
-  if (e == hipSuccess && lds > 64 * 1024 && opt_in_lds(p->func, lds) != RL_OK) e = hipErrorInvalidValue;
   if (e != hipSuccess) {
     if (p->module) (void)hipModuleUnload(p->module);
     delete p;
     return hip_fail(e, "loading the compiled GEMM kernel");
+  }
+  // opt in to the plan's LDS size and read back what the runtime grants: a refusal is reported
+  // here, with text, and not by the first launch
+  rc = opt_in_lds(p->func, lds, &p->lds_limit);
+  if (rc) {
+    (void)hipModuleUnload(p->module);
+    delete p;
+    return rc;
   }
   p->vgprs = metadata_int(code, ".vgpr_count");
   p->agprs = metadata_int(code, ".agpr_count");
@@ -635,12 +702,14 @@ int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* co
 
 int rl_gemm_plan_function(const rl_gemm_plan* plan, rl_function* out) {
   if (!plan || !out) return fail(RL_ERR_INVALID_ARG, "rl_gemm_plan_function: NULL argument");
+  std::shared_lock<std::shared_mutex> in_flight(g_plans_rw);
   if (!plan->func) return fail(RL_ERR_INVALID_ARG, "plan was released by rl_gemm_plans_clear");
   *out = plan->func;
   return RL_OK;
 }
 
 int rl_gemm_plan_lds_bytes(const rl_gemm_plan* plan) { return plan ? plan->lds_bytes : 0; }
+int rl_gemm_plan_lds_limit(const rl_gemm_plan* plan) { return plan ? plan->lds_limit : 0; }
 int rl_gemm_plan_threads(const rl_gemm_plan* plan) { return plan ? plan->threads : 0; }
 
 int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int* sgprs,
@@ -655,7 +724,11 @@ int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int
 }
 
 int rl_gemm_plans_clear(void) {
+  READY_OR_RETURN();
   std::lock_guard<std::mutex> lock(g_mutex);
+  std::unique_lock<std::shared_mutex> no_launches(g_plans_rw);
+  // launches enqueued earlier may still be running the code that is about to be unloaded
+  HIP_TRY(hipDeviceSynchronize());
   int rc = RL_OK;
   for (auto& kv : g_plans) {
     if (kv.second->module) {
@@ -673,6 +746,8 @@ int rl_gemm_plans_clear(void) {
 int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
                         int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream) {
   if (!plan) return fail(RL_ERR_INVALID_ARG, "plan is NULL");
+  READY_OR_RETURN();
+  std::shared_lock<std::shared_mutex> in_flight(g_plans_rw);
   if (!plan->func) return fail(RL_ERR_INVALID_ARG, "plan was released by rl_gemm_plans_clear");
   const rl_gemm_config& c = plan->cfg;
   if (M < 0 || N < 0 || K < 0) return fail(RL_ERR_INVALID_ARG, "negative dimension (M=%d N=%d K=%d)", M, N, K);

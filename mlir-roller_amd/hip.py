@@ -160,6 +160,7 @@ _SIGNATURES = {
     "rl_gemm_plan_create": ([C.POINTER(_GemmConfigC), C.POINTER(C.c_void_p), C.POINTER(C.c_float)], C.c_int),
     "rl_gemm_plan_function": ([C.c_void_p, C.POINTER(C.c_void_p)], C.c_int),
     "rl_gemm_plan_lds_bytes": ([C.c_void_p], C.c_int),
+    "rl_gemm_plan_lds_limit": ([C.c_void_p], C.c_int),
     "rl_gemm_plan_threads": ([C.c_void_p], C.c_int),
     "rl_gemm_plan_resources": ([C.c_void_p] + [C.POINTER(C.c_int)] * 5, C.c_int),
     "rl_gemm_plans_clear": ([], C.c_int),
@@ -407,16 +408,42 @@ class Module:
             pass
 
 
+class Ptr:
+    """A raw device address as a kernel argument (``dA.data.ptr`` in the reference,
+    roller.py:548): always passed as an 8-byte pointer, whatever its value (NULL included)."""
+
+    __slots__ = ("address",)
+
+    def __init__(self, address: int):
+        address = int(address)
+        if not 0 <= address < 2**64:
+            raise ValueError(f"device address {address:#x} does not fit 64 bits")
+        self.address = address
+
+    def __repr__(self) -> str:
+        return f"Ptr({self.address:#x})"
+
+
 def _pack_arg(a):
+    """One kernel argument as the ctypes object whose storage ``hipModuleLaunchKernel`` reads.
+    The width is decided by the argument's type, never by its value: ``DeviceArray``, ``Ptr``
+    and ``c_void_p`` are 8-byte pointers; a Python or numpy integer is a 4-byte ``int``
+    (``OverflowError`` if it does not fit -- use ``ctypes.c_long`` for a 64-bit parameter and
+    ``Ptr`` for an address); a float is a 4-byte ``float``; ctypes scalars pass through."""
     if isinstance(a, DeviceArray):
         return C.c_void_p(a.ptr)
+    if isinstance(a, Ptr):
+        return C.c_void_p(a.address)
     if isinstance(a, (C._SimpleCData,)):
         return a
+    if isinstance(a, (bool, np.bool_)):
+        raise TypeError("cannot pass a bool to a kernel; use an int")
     if isinstance(a, (int, np.integer)):
-        # Pointers arrive as Python ints (``dA.data.ptr`` in the reference); anything that does
-        # not fit an int32 is taken to be an address.
         v = int(a)
-        return C.c_int(v) if -2**31 <= v < 2**31 else C.c_void_p(v)
+        if not -2**31 <= v < 2**31:
+            raise OverflowError(f"{v} does not fit a 32-bit int kernel parameter; pass ctypes.c_long(...) for a "
+                                "64-bit integer or hip.Ptr(...) for a device address")
+        return C.c_int(v)
     if isinstance(a, (float, np.floating)):
         return C.c_float(float(a))
     raise TypeError(f"cannot pass {type(a).__name__} to a kernel")
@@ -458,6 +485,16 @@ def precompile(cfg: GemmConfig) -> int:
     return size.value
 
 
+def _address(x) -> int:
+    """Device address of a matrix argument of the typed GEMM entry points (their ctypes
+    signatures declare pointers, so an int is never mistaken for anything else)."""
+    if isinstance(x, DeviceArray):
+        return x.ptr
+    if isinstance(x, Ptr):
+        return x.address
+    return int(x)
+
+
 class GemmPlan:
     """One compiled and loaded instance of the kernel template (``rl_gemm_plan``)."""
 
@@ -470,6 +507,7 @@ class GemmPlan:
         self.handle = p.value
         self.compile_ms = float(ms.value)
         self.lds_bytes = lib().rl_gemm_plan_lds_bytes(self.handle)
+        self.lds_limit = lib().rl_gemm_plan_lds_limit(self.handle)
         self.threads = lib().rl_gemm_plan_threads(self.handle)
 
     @property
@@ -485,7 +523,7 @@ class GemmPlan:
 
     def launch(self, A, B, Cm, M: int, N: int, K: int, lda: Optional[int] = None,
                ldb: Optional[int] = None, ldc: Optional[int] = None, stream=None) -> None:
-        ptr = lambda x: x.ptr if isinstance(x, DeviceArray) else int(x)
+        ptr = _address
         width_b = K if self.cfg.trans_b else N
         check(lib().rl_gemm_plan_launch(self.handle, ptr(A), ptr(B), ptr(Cm), M, N, K,
                                         K if lda is None else lda, width_b if ldb is None else ldb,
@@ -496,7 +534,7 @@ def gemm_f32(cfg: GemmConfig, A, B, Cm, M: int, N: int, K: int, lda=None, ldb=No
              stream=None) -> None:
     """``rl_gemm_f32``: plan lookup (JIT on first use) + launch in one call."""
     init()
-    ptr = lambda x: x.ptr if isinstance(x, DeviceArray) else int(x)
+    ptr = _address
     c = cfg.to_c()
     width_b = K if cfg.trans_b else N
     check(lib().rl_gemm_f32(C.byref(c), ptr(A), ptr(B), ptr(Cm), M, N, K,

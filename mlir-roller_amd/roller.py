@@ -22,7 +22,7 @@ from typing import Optional, Tuple
 import numpy as np
 
 from . import hip
-from .analyze import MatmulConfig, TileDict, get_roller_hints, split_block_over_waves
+from .analyze import MatmulConfig, TileDict, get_roller_hints, loads_go_direct_to_lds, split_block_over_waves
 from .arch import MI355X
 from .hip import DeviceArray, Event, GemmConfig, GemmPlan
 from .utils import get_block_dims
@@ -66,14 +66,19 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
     # At full depth and width the global loads go straight to LDS (swizzled A rows, no padding)
     # whenever both operand tiles are whole waves of 16-byte units and the K step is a power of
     # two (the swizzle is an XOR).
-    direct = int(stages == 3 and vec == 4 and bk & (bk - 1) == 0
-                 and (bm * bk // 4) % 64 == 0 and (bk * bn // 4) % 64 == 0)
+    direct = int(loads_go_direct_to_lds(config, (bm, bn), bk, stages))
     # otherwise (bk + pad)/4 odd keeps the 128-bit reads of LDS-A free of bank conflicts
     pad_a = 0 if direct else (4 if (bk // 4) % 2 == 0 else 0)
-    # a transposed second operand sits in LDS like A and wants the same padding, LDS permitting
+    # a transposed second operand sits in LDS like A and wants the same padding
     pad_b = pad_a if trans_b else 0
-    if pad_b and min(stages, 2) * (bm * (bk + pad_a) + bn * (bk + pad_b)) * 4 > MI355X().lds_bytes:
+    # Padding is an optimisation, fitting the CU is not: a hint whose policy ran for another depth
+    # or layout may leave no room for it.
+    lds_cap = MI355X().lds_bytes
+    footprint = lambda pa, pb: min(stages, 2) * (bm * (bk + pa) + (bn * (bk + pb) if trans_b else bk * (bn + pb))) * 4
+    if pad_b and footprint(pad_a, pad_b) > lds_cap:
         pad_b = 0
+    if pad_a and footprint(pad_a, pad_b) > lds_cap:
+        pad_a = 0
     return GemmConfig(
         bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi, stages=stages, pad_a=pad_a, pad_b=pad_b, vec=vec,
         edge=0 if (M % bm == 0 and N % bn == 0 and K % bk == 0) else 1,

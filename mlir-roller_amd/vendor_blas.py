@@ -16,7 +16,7 @@ from pathlib import Path
 from typing import Optional
 
 from . import hip
-from .hip import DeviceArray
+from .hip import _address
 
 OPERATION_NONE = 111          # rocblas_operation_none
 STATUS_SUCCESS = 0            # rocblas_status_success
@@ -61,7 +61,7 @@ class RocBLAS:
     def sgemm_row_major(self, A, B, Cm, M: int, N: int, K: int, lda: Optional[int] = None,
                         ldb: Optional[int] = None, ldc: Optional[int] = None) -> None:
         """Enqueues ``C = A @ B`` for row-major fp32 device matrices (pointers or ``DeviceArray``)."""
-        ptr = lambda x: x.ptr if isinstance(x, DeviceArray) else int(x)
+        ptr = _address
         self._check(self._lib.rocblas_sgemm(
             self._handle, OPERATION_NONE, OPERATION_NONE, N, M, K, C.byref(self._one),
             ptr(B), N if ldb is None else ldb, ptr(A), K if lda is None else lda,

@@ -207,3 +207,53 @@ def test_vendor_library_missing_is_reported_not_fatal(tmp_path):
     from mlir_roller_amd.vendor_blas import RocBLAS, VendorBlasError
     with pytest.raises(VendorBlasError, match="cannot load rocBLAS"):
         RocBLAS(library=str(tmp_path / "librocblas.so"))
+
+
+@pytest.mark.parametrize("depth", [1, 2, 3])
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_every_hint_fits_the_kernel_at_every_pipeline_depth(hip_lib, depth, trans_b):
+    # the policy's LDS model follows the depth: padded rows and two buffers at depth 2, swizzled
+    # unpadded rows at depth 3; no emitted hint may be refused by the library's own check
+    from mlir_roller_amd import hip
+    shapes = list(bm.README_SHAPES) + [(3000, 5000, 1536), (1000, 1000, 1000), (1022, 1018, 1002), (37, 53, 29)]
+    for shape in shapes:
+        cfg = MatmulConfig(*shape, 32)
+        hints = get_roller_hints(cfg, MI355X(), 20, pipeline_depth=depth)
+        assert hints, shape
+        for hint in hints:
+            g = roller.hint_to_gemm_config(cfg, hint, depth, trans_b=trans_b)
+            lds, threads = hip.config_check(g)
+            assert lds <= 160 * 1024 and threads == hint.threads
+            if not trans_b:
+                assert lds == min(depth, 2) * hint.smem_cost, (shape, hint)   # the model is exact, not just safe
+
+
+def test_a_hint_ranked_for_another_depth_still_fits(hip_lib):
+    # Compiler(config, hint, 2) with a hint that the policy sized for depth 3: padding is dropped
+    # where it would overflow the CU's LDS
+    from mlir_roller_amd import hip
+    cfg = MatmulConfig(2048, 2048, 2048, 32)
+    for hint in get_roller_hints(cfg, MI355X(), 20, pipeline_depth=3):
+        for trans_b in (False, True):
+            hip.config_check(roller.hint_to_gemm_config(cfg, hint, 2, trans_b=trans_b))
+
+
+def test_kernel_arguments_are_typed_by_type_not_by_value():
+    import ctypes as C
+    from mlir_roller_amd import hip
+    assert C.sizeof(hip._pack_arg(hip.Ptr(0))) == 8 and hip._pack_arg(hip.Ptr(0)).value is None   # NULL stays a pointer
+    assert C.sizeof(hip._pack_arg(hip.Ptr(4096))) == 8
+    for small in (0, 7, -1, 2**31 - 1, np.int64(12)):
+        packed = hip._pack_arg(small)
+        assert isinstance(packed, C.c_int) and C.sizeof(packed) == 4      # a bare int is never a pointer
+    for wide in (2**31, 2**40, 0x7F0000000000, -2**31 - 1):
+        with pytest.raises(OverflowError):
+            hip._pack_arg(wide)
+    assert isinstance(hip._pack_arg(C.c_long(2**40)), C.c_long)
+    assert isinstance(hip._pack_arg(1.5), C.c_float)
+    with pytest.raises(TypeError):
+        hip._pack_arg(True)
+    with pytest.raises(TypeError):
+        hip._pack_arg("x")
+    with pytest.raises(ValueError):
+        hip.Ptr(-1)
