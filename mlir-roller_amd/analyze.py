@@ -229,10 +229,10 @@ MAX_BLOCKS_PER_WAVE = 32
 
 def split_block_over_waves(block_tile: List[int], waves: int, rstep: int, arch: TileDevice, shapes=None):
     """Wave tile ``[wm, wn]`` and MFMA size for a block tile computed by ``waves`` wavefronts,
-    or None.  A wave tile must be a grid of MFMA blocks whose column count the kernel reads
-    with one vector load (1, 2 or a multiple of 4 blocks), and the reduce step must hold whole
-    128-bit fragment reads (4 * wave / mi elements of k), and a wave owns at most
-    ``MAX_BLOCKS_PER_WAVE`` blocks.  The larger instruction is preferred;
+    or None.  A wave tile must be a grid of MFMA blocks (any column count: the kernel reads the
+    second operand with the widest of 128-, 64- and 32-bit loads that divides it), the reduce
+    step must hold whole 128-bit fragment reads (4 * wave / mi elements of k), and a wave owns at
+    most ``MAX_BLOCKS_PER_WAVE`` blocks.  The larger instruction is preferred;
     among its wave tiles the most square wins, wider before taller."""
     m, n = block_tile
     for shape in (arch.mfma_shapes if shapes is None else shapes):
@@ -247,10 +247,7 @@ def split_block_over_waves(block_tile: List[int], waves: int, rstep: int, arch: 
             wm, wn = m // rows, n // cols
             if wm % mi or wn % mi:
                 continue
-            col_blocks = wn // mi
-            if not (col_blocks in (1, 2) or col_blocks % 4 == 0):
-                continue
-            if (wm // mi) * col_blocks > MAX_BLOCKS_PER_WAVE:
+            if (wm // mi) * (wn // mi) > MAX_BLOCKS_PER_WAVE:
                 continue
             key = (wm + wn, -wn)
             if best is None or key < best[0]:
@@ -265,7 +262,7 @@ class Policy:
 
     # tile sizes offered in addition to the exact divisors of a dimension
     SIMT_LADDER = (2, 4, 8, 16, 32)
-    MFMA_LADDER = (16, 32, 64, 128, 256, 512)
+    MFMA_LADDER = (16, 32, 48, 64, 96, 128, 160, 192, 256, 320, 384, 512)
     # registers per lane the MFMA kernel needs besides its accumulators and operand fragments:
     # addresses, loop state, buffer resources (measured: 40-60)
     REG_OVERHEAD = 50
@@ -342,18 +339,19 @@ class Policy:
         cores.  The busiest CU works through ceil(grid / CUs) tiles one after another.  A tile
         costs the larger of its MFMA time at the CU's share of the matrix peak and its traffic at
         the CU's share of the memory bandwidth.  MFMA time is divided by an issue efficiency that
-        falls with the operand traffic per FLOP, (1/m + 1/n): fitted to measurements on MI355X
-        (about 0.95 for 256x256 tiles, 0.81 for 32x64).  A fixed cost per tile covers filling the
+        falls with the operand traffic per FLOP, (1/m + 1/n); its two constants are fields of the
+        device model, fitted to a committed sweep (``calibrate.py``).  A fixed cost per tile covers filling the
         pipeline and draining the accumulators."""
         a, cfg = self.arch, self.matmul_config
         m, n = td.block_tile
         cu_flops = a.peak_matrix_tflops * 1e12 / a.compute_max_core
         cu_bw = a.bandwidth[0] * 1e9 / a.compute_max_core
         k_steps = -(-cfg.K // td.rstep)  # the kernel runs whole K steps also where K is ragged
-        efficiency = max(0.972 - 3.456 * (1.0 / m + 1.0 / n), 0.05)
+        base, slope = a.mfma_efficiency
+        efficiency = max(base - slope * (1.0 / m + 1.0 / n), 0.05)
         t_mfma = 2.0 * m * n * k_steps * td.rstep / (cu_flops * efficiency)
         t_mem = td.traffic / cu_bw
-        t_fixed = 1.0e-6 + m * n * cfg.el_bytes / cu_bw
+        t_fixed = a.tile_fixed_seconds + m * n * cfg.el_bytes / cu_bw
         tiles_per_cu = -(-td.grid_size // a.compute_max_core)
         return tiles_per_cu * (max(t_mfma, t_mem) + t_fixed)
 

@@ -51,6 +51,11 @@ class TileDevice:
     peak_matrix_tflops: float = 0.0
     # peak engine clock, MHz (0 = unknown)
     clock_mhz: int = 0
+    # ranking model of devices with matrix cores (``Policy.estimate_seconds``): the matrix pipe's
+    # issue efficiency on a block tile [m, n] is base - slope * (1/m + 1/n), and every tile pays
+    # ``tile_fixed_seconds`` (pipeline fill) on top of storing its results
+    mfma_efficiency: Tuple[float, float] = (1.0, 0.0)
+    tile_fixed_seconds: float = 0.0
 
     def get_avaliable_tensorintrin_shapes(self) -> List[Tuple[int, int, int]]:
         """Matrix-instruction shapes of the device (name kept from the reference, arch.py:36)."""
@@ -119,6 +124,10 @@ class MI355X(TileDevice):
     xcd_count: int = 8
     peak_matrix_tflops: float = 157.3
     clock_mhz: int = 2400
+    # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
+    # (a test refits it): about 0.95 for 256x256 tiles, 0.81 for 32x64
+    mfma_efficiency: Tuple[float, float] = (0.972, 3.456)
+    tile_fixed_seconds: float = 1.0e-6
     smem_cap: int = field(init=False)
     max_smem_usage: int = field(init=False)
 

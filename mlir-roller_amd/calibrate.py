@@ -1,0 +1,260 @@
+"""Calibration of the MI355X ranking model against measurements.
+
+    python -m mlir_roller_amd.calibrate measure [--out FILE] [--topk 48] [--shapes M0 M10 1024x1024x1024 ...]
+    python -m mlir_roller_amd.calibrate fit     [--data FILE]
+    python -m mlir_roller_amd.calibrate check   [--data FILE] [--topk 4]
+
+The reference ranks block tiles by ``(traffic + 1) * num_wave`` and then simply tries its first
+twenty (/root/reference/src/analyze.py:241-255, benchmark.py:10).  Here the ranking is a roofline
+estimate (``Policy.estimate_seconds``) whose constants live in ``arch.MI355X`` and are fitted to a
+sweep of the kernel on the device, so that few hints have to be tried:
+
+``measure``  (needs the GPU) times, for every shape, the kernels of the policy's first ``topk``
+             hints and writes one record per (shape, kernel) -- the data set committed under
+             ``calibration/``;
+``fit``      (no GPU) refits the constants from such a data set: per (shape, block tile) the best
+             measured time gives an observed MFMA issue efficiency, and ordinary least squares of
+             that efficiency against ``1/m + 1/n`` gives ``mfma_efficiency = (base, slope)``;
+``check``    (no GPU) replays the policy on the data set: where does the measured best sit in the
+             policy's order, and how far from it is the best of the first ``topk`` hints.
+
+A CPU test refits the committed data set and compares the result with the committed constants,
+so the two cannot drift apart.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import sys
+from pathlib import Path
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple
+
+from .analyze import DEFAULT_PIPELINE_DEPTH, MatmulConfig, Policy, TileDict, get_roller_hints
+from .arch import MI355X, TileDevice
+
+DATA_DIR = Path(__file__).resolve().parent / "calibration"
+DEFAULT_DATA = DATA_DIR / "mi355x_f32.json"
+
+# the fourteen benchmark shapes, the ragged named configuration and three mid-size cubes
+SHAPES: Dict[str, Tuple[int, int, int]] = {f"M{i}": s for i, s in enumerate([
+    (2048, 2048, 2048), (2048, 2048, 8192), (2048, 4096, 2048), (2048, 4096, 4096), (2048, 8192, 2048),
+    (2048, 8192, 4096), (2048, 8192, 8192), (4096, 2048, 2048), (4096, 4096, 8192), (4096, 8192, 2048),
+    (4096, 8192, 4096), (8192, 2048, 8192), (8192, 4096, 2048), (8192, 4096, 4096)])}
+SHAPES.update({"cfg4": (3000, 5000, 1536), "1024x1024x1024": (1024, 1024, 1024),
+               "1536x1536x1536": (1536, 1536, 1536), "1000x1000x1000": (1000, 1000, 1000)})
+
+
+def shape_of(name: str) -> Tuple[int, int, int]:
+    if name in SHAPES:
+        return SHAPES[name]
+    dims = tuple(int(v) for v in name.lower().split("x"))
+    if len(dims) != 3 or min(dims) <= 0:
+        raise ValueError(f"unknown shape {name!r}")
+    return dims  # type: ignore[return-value]
+
+
+# ---------------------------------------------------------------------------------------------
+# the model, restated on plain numbers so that a fit can evaluate it without building TileDicts
+# ---------------------------------------------------------------------------------------------
+
+def ideal_tile_seconds(m: int, n: int, K: int, rstep: int, arch: TileDevice) -> float:
+    """MFMA time of one block tile over the whole of K at a CU's share of the matrix peak."""
+    k_steps = -(-K // rstep)
+    return 2.0 * m * n * k_steps * rstep / (arch.peak_matrix_tflops * 1e12 / arch.compute_max_core)
+
+
+def fixed_tile_seconds(m: int, n: int, arch: TileDevice, el_bytes: int = 4) -> float:
+    """The part of a tile's time that does not scale with K (pipeline fill, storing C)."""
+    return arch.tile_fixed_seconds + m * n * el_bytes / (arch.bandwidth[0] * 1e9 / arch.compute_max_core)
+
+
+def observed_efficiency(rec: dict, arch: TileDevice) -> Optional[float]:
+    """MFMA issue efficiency that one measurement implies under the model's structure:
+    tiles_per_cu * (ideal / efficiency + fixed) = measured."""
+    M, N, K = rec["shape"]
+    m, n = rec["block_tile"]
+    tiles = (-(-M // m)) * (-(-N // n))
+    per_cu = -(-tiles // arch.compute_max_core)
+    busy = rec["ms"] * 1e-3 / per_cu - fixed_tile_seconds(m, n, arch)
+    if busy <= 0:
+        return None
+    return ideal_tile_seconds(m, n, K, rec["rstep"], arch) / busy
+
+
+def best_per_block_tile(records: Iterable[dict]) -> List[dict]:
+    """The fastest record of every (shape, block tile): wave split, instruction and K step are
+    second-order choices that the fit of the tile-level efficiency must not see."""
+    best: Dict[tuple, dict] = {}
+    for r in records:
+        key = (tuple(r["shape"]), tuple(r["block_tile"]))
+        if key not in best or r["ms"] < best[key]["ms"]:
+            best[key] = r
+    return [best[k] for k in sorted(best)]
+
+
+def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
+    """Least-squares ``efficiency = base - slope * (1/m + 1/n)`` over the best record of every
+    (shape, block tile) whose tile grid fills at least three quarters of its last round of CUs
+    (a sparse last round measures the tail, not the tile).  Deterministic: closed-form normal
+    equations, records in sorted order."""
+    arch = arch or MI355X()
+    xs, ys = [], []
+    for r in best_per_block_tile(records):
+        M, N, _ = r["shape"]
+        m, n = r["block_tile"]
+        tiles = (-(-M // m)) * (-(-N // n))
+        last_round = tiles % arch.compute_max_core or arch.compute_max_core
+        if M % m or N % n or last_round < 0.75 * arch.compute_max_core:
+            continue
+        eff = observed_efficiency(r, arch)
+        if eff is None or not 0.3 < eff < 1.05:
+            continue
+        xs.append(1.0 / m + 1.0 / n)
+        ys.append(eff)
+    if len(xs) < 3:
+        raise ValueError(f"only {len(xs)} usable records; need at least 3 distinct block tiles")
+    n_pts = float(len(xs))
+    sx, sy = math.fsum(xs), math.fsum(ys)
+    sxx, sxy = math.fsum(x * x for x in xs), math.fsum(x * y for x, y in zip(xs, ys))
+    slope = (n_pts * sxy - sx * sy) / (n_pts * sxx - sx * sx)
+    base = (sy - slope * sx) / n_pts
+    resid = [y - (base + slope * x) for x, y in zip(xs, ys)]
+    return {"mfma_efficiency": (round(base, 3), round(-slope, 2)), "base": base, "slope": -slope, "points": len(xs),
+            "rms_residual": math.sqrt(math.fsum(e * e for e in resid) / n_pts)}
+
+
+# ---------------------------------------------------------------------------------------------
+# replaying the policy on a data set
+# ---------------------------------------------------------------------------------------------
+
+def _key_of_hint(hint: TileDict) -> tuple:
+    return (tuple(hint.block_tile), tuple(hint.wave_tile), hint.mfma, hint.rstep)
+
+
+def _key_of_record(rec: dict) -> tuple:
+    return (tuple(rec["block_tile"]), tuple(rec["wave_tile"]), rec["mfma"], rec["rstep"])
+
+
+def check(records: Sequence[dict], arch: Optional[TileDevice] = None, topk: int = 4, depth: int = DEFAULT_PIPELINE_DEPTH) -> List[dict]:
+    """Per shape of the data set: rank (in the policy's current order) of the fastest measured
+    kernel, time of the first hint over the fastest, time of the best of the first ``topk`` hints
+    over the fastest, and how many of those first hints the data set has no measurement for."""
+    arch = arch or MI355X()
+    by_shape: Dict[tuple, Dict[tuple, float]] = {}
+    for r in records:
+        by_shape.setdefault(tuple(r["shape"]), {})[_key_of_record(r)] = r["ms"]
+    rows = []
+    for shape in sorted(by_shape):
+        measured = by_shape[shape]
+        hints = get_roller_hints(MatmulConfig(*shape, 32), arch, topk=200, pipeline_depth=depth)
+        order = [_key_of_hint(h) for h in hints]
+        fastest_key = min(measured, key=measured.get)
+        fastest = measured[fastest_key]
+        head = [measured.get(k) for k in order[:topk]]
+        known = [t for t in head if t is not None]
+        rows.append({
+            "shape": list(shape),
+            "fastest_ms": fastest,
+            "fastest_rank": order.index(fastest_key) + 1 if fastest_key in order else None,
+            "top1_over_fastest": (head[0] / fastest) if head and head[0] is not None else None,
+            "topk_over_fastest": (min(known) / fastest) if known else None,
+            "unmeasured_in_topk": sum(t is None for t in head),
+        })
+    return rows
+
+
+# ---------------------------------------------------------------------------------------------
+# measuring (GPU)
+# ---------------------------------------------------------------------------------------------
+
+def measure(shape_names: Sequence[str], topk: int, depth: int = DEFAULT_PIPELINE_DEPTH, chunk: int = 8,
+            say=lambda *a: print(*a, file=sys.stderr, flush=True)) -> dict:
+    import numpy as np
+
+    from . import hip
+    from .hip import DeviceArray, GemmPlan, Stream
+    from .roller import hint_to_gemm_config, make_inputs
+    from .tuner import time_candidates
+
+    hip.init(0)
+    props = hip.device_info()
+    arch = MI355X.from_device(props)
+    stream = Stream()
+    records: List[dict] = []
+    for name in shape_names:
+        shape = shape_of(name)
+        M, N, K = shape
+        cfg = MatmulConfig(M, N, K, 32)
+        A, B = make_inputs(cfg, 0, "uniform")
+        bufs = (DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray.zeros((M, N)))
+        del A, B
+        hints = get_roller_hints(cfg, arch, topk=topk, pipeline_depth=depth)
+        cands = []
+        for rank, hint in enumerate(hints, 1):
+            try:
+                g = hint_to_gemm_config(cfg, hint, depth)
+                cands.append((rank, hint, g, GemmPlan(g)))
+            except Exception as e:  # a hint the device refuses is simply not part of the data
+                say(f"[calibrate] {name} hint {rank} skipped: {e}")
+        for i in range(0, len(cands), chunk):
+            part = cands[i:i + chunk]
+            times = time_candidates([c[3] for c in part], bufs, shape, stream=stream)
+            for (rank, hint, g, _), ms in zip(part, times):
+                records.append({"shape": list(shape), "block_tile": list(hint.block_tile), "wave_tile": list(hint.wave_tile),
+                                "mfma": hint.mfma, "rstep": hint.rstep, "threads": hint.threads, "edge": g.edge,
+                                "direct": g.direct, "rank_when_measured": rank, "ms": round(ms, 6)})
+        best = min((r for r in records if r["shape"] == list(shape)), key=lambda r: r["ms"])
+        say(f"[calibrate] {name} {shape}: {len(cands)} kernels, best {best['ms']:.4f} ms "
+            f"({2.0 * M * N * K / best['ms'] / 1e9:.1f} TFLOP/s) rank {best['rank_when_measured']} {best['block_tile']}/{best['wave_tile']}/mi{best['mfma']}/k{best['rstep']}")
+        for b in bufs:
+            b.free()
+    return {"device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units,
+                       "clock_khz": props.clock_khz},
+            "pipeline_depth": depth, "protocol": "per kernel: best of 2 alternating batches of 8 launches behind a 40 ms clock ramp, HIP events on the launch stream",
+            "records": records}
+
+
+def load(path: Path = DEFAULT_DATA) -> dict:
+    return json.loads(Path(path).read_text())
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description="fit / check the MI355X ranking model of the rTile policy")
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    m = sub.add_parser("measure")
+    m.add_argument("--out", default=str(DEFAULT_DATA))
+    m.add_argument("--topk", type=int, default=48)
+    m.add_argument("--shapes", nargs="*", default=list(SHAPES))
+    f = sub.add_parser("fit")
+    f.add_argument("--data", default=str(DEFAULT_DATA))
+    c = sub.add_parser("check")
+    c.add_argument("--data", default=str(DEFAULT_DATA))
+    c.add_argument("--topk", type=int, default=4)
+    args = ap.parse_args(argv)
+
+    if args.cmd == "measure":
+        data = measure(args.shapes, args.topk)
+        out = Path(args.out)
+        out.parent.mkdir(parents=True, exist_ok=True)
+        out.write_text(json.dumps(data, separators=(",", ":")).replace('},{"shape"', '},\n{"shape"'))
+        print(f"{len(data['records'])} records written to {out}")
+        return 0
+    data = load(Path(args.data))
+    if args.cmd == "fit":
+        res = fit(data["records"])
+        now = MI355X().mfma_efficiency
+        print(f"fitted mfma_efficiency = {res['mfma_efficiency']} from {res['points']} block tiles "
+              f"(rms residual {res['rms_residual']:.4f}); arch.MI355X has {tuple(now)}")
+        return 0
+    rows = check(data["records"], topk=args.topk)
+    for r in rows:
+        fmt = lambda v: "-" if v is None else f"{v:.4f}"
+        print(f"{'x'.join(map(str, r['shape'])):>18}  fastest rank {r['fastest_rank']!s:>4}  top1/fastest {fmt(r['top1_over_fastest'])}  "
+              f"top{args.topk}/fastest {fmt(r['topk_over_fastest'])}  unmeasured {r['unmeasured_in_topk']}")
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

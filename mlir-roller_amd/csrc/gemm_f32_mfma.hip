@@ -131,7 +131,9 @@
 #define TN (WN / MI)
 #define KG (64 / MI)       /* lane groups along k inside one MFMA (= its k extent) */
 #define KSUPER (4 * KG)    /* k covered by the four MFMAs fed from one 128-bit A read */
-#define VN (TN >= 4 ? 4 : TN)
+/* column blocks that one B read feeds: the widest of 4, 2, 1 that divides TN (TN = 3, 5: dword
+ * reads; 6, 10: 64-bit reads; multiples of 4: 128-bit reads) */
+#define VN (TN % 4 == 0 ? 4 : (TN % 2 == 0 ? 2 : 1))
 #define NVB (TN / VN)
 #define LDA_S (BK + PAD_A)
 #if TRANS_B
@@ -162,7 +164,6 @@
 static_assert(MI == 32 || MI == 16, "MI selects v_mfma_f32_32x32x2_f32 or v_mfma_f32_16x16x4_f32");
 static_assert(BM % WM == 0 && BN % WN == 0, "wave tile must divide block tile");
 static_assert(WM % MI == 0 && WN % MI == 0, "MFMA block must divide wave tile");
-static_assert(TN == 1 || TN == 2 || TN % 4 == 0, "column blocks per wave: 1, 2 or a multiple of 4");
 static_assert(TM * TN <= 32, "at most 32 MFMA blocks per wave: beyond that the accumulator array is no longer kept in registers");
 static_assert(BK % KSUPER == 0, "BK must be a multiple of 4*(64/MI)");
 static_assert(PAD_A % 4 == 0 && PAD_B % 4 == 0, "LDS rows stay 16-byte aligned");

@@ -115,8 +115,6 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
   if (c.wm % c.mi || c.wn % c.mi)
     return fail(RL_ERR_INVALID_ARG, "MFMA block %d does not divide wave tile %dx%d", c.mi, c.wm, c.wn);
   const int tn = c.wn / c.mi;
-  if (!(tn == 1 || tn == 2 || tn % 4 == 0))
-    return fail(RL_ERR_INVALID_ARG, "wn/mi must be 1, 2 or a multiple of 4, got %d", tn);
   if ((c.wm / c.mi) * tn > 32)
     return fail(RL_ERR_INVALID_ARG, "wave tile %dx%d is %d MFMA blocks of %d; at most 32 are kept in registers", c.wm, c.wn, (c.wm / c.mi) * tn, c.mi);
   if (c.bn % 4) return fail(RL_ERR_INVALID_ARG, "bn must be a multiple of 4");

@@ -495,6 +495,38 @@ def _address(x) -> int:
     return int(x)
 
 
+def _precompile_worker(cfg_values: tuple) -> tuple:
+    cfg = GemmConfig(*cfg_values)
+    try:
+        return cfg_values, precompile(cfg), ""
+    except HipError as e:
+        return cfg_values, 0, str(e)
+
+
+def precompile_many(configs: Sequence[GemmConfig], jobs: Optional[int] = None) -> dict:
+    """Fills the on-disk cache for ``configs`` with ``jobs`` worker processes (hiprtc is
+    single-threaded and needs no GPU; default: the CPUs this process may run on, at most 16).
+    Returns ``{config: error text}`` for the ones that failed; the rest are in the cache."""
+    import concurrent.futures as cf
+
+    todo = list(dict.fromkeys(configs))
+    if jobs is None:
+        jobs = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
+    values = [tuple(getattr(c, f.name) for f in fields(c)) for c in todo]
+    failed = {}
+    if jobs <= 1 or len(todo) <= 1:
+        results = map(_precompile_worker, values)
+    else:
+        pool = cf.ProcessPoolExecutor(max_workers=min(jobs, len(todo)))
+        results = pool.map(_precompile_worker, values, chunksize=1)
+    for vals, _, err in results:
+        if err:
+            failed[GemmConfig(*vals)] = err
+    if jobs > 1 and len(todo) > 1:
+        pool.shutdown()
+    return failed
+
+
 class GemmPlan:
     """One compiled and loaded instance of the kernel template (``rl_gemm_plan``)."""
 

