@@ -65,15 +65,17 @@ typedef struct rl_gemm_config {
   int bk;          /* K step                <- hint.rstep                            */
   int wm, wn;      /* wave tile             <- 64 lanes x hint.thread_tile           */
   int mi;          /* 32: v_mfma_f32_32x32x2_f32, 16: v_mfma_f32_16x16x4_f32        */
-  int stages;      /* pipeline depth 1..3   <- pipeline_depth (2 LDS buffers from 2) */
+  int stages;      /* pipeline depth 1..5   <- pipeline_depth: 1, 2, 2, 3, 4 LDS buffers;
+                      3 adds a register stage, 4 and 5 need direct=1                 */
   int pad_a, pad_b;/* LDS row padding in floats (multiples of 4)                     */
   int vec;         /* 4: 128-bit global accesses, 1: dword accesses (any K, N, ld)   */
-  int edge;        /* 1: ragged tiles predicated, 0: bm|M, bn|N, bk|K required       */
+  int edge;        /* 1: ragged tiles predicated (any M, N, K), 2: M and N may be ragged,
+                      bk|K required, 0: bm|M, bn|N, bk|K required                     */
   int swz;         /* bit0: XCD-contiguous tile order, bit1: panel walk              */
   int group;       /* panel height in tiles (reference: panel-width=8, roller.py:338)*/
   int accum;       /* 0: C = A*B, 1: C += A*B (linalg.matmul semantics, roller.py:62)*/
   int direct;      /* 1: global loads write LDS directly (no staging registers, swizzled
-                      A rows); needs stages=3, vec=4, pad_a=pad_b=0, bk a power of 2 */
+                      A rows); needs stages>=3, vec=4, pad_a=pad_b=0, bk a power of 2 */
   int trans_b;     /* 1: the second operand is Bt[N][ldb>=K], C = A*Bt^T (the [spatial, reduce]
                       layout of MatmulConfig.get_input_shapes, src/analyze.py:33-41); pad_b then
                       pads the K-contiguous rows of its LDS tile like pad_a                   */
@@ -142,7 +144,7 @@ int rl_sync(void);
 const char* rl_gemm_template_source(void);
 
 /* Checks cfg against the template's constraints without compiling.  *lds_bytes (may be NULL)
- * receives the dynamic LDS size = min(stages,2) * (bm*(bk+pad_a) + bk*(bn+pad_b)) * 4
+ * receives the dynamic LDS size = buffers(stages) * (bm*(bk+pad_a) + bk*(bn+pad_b)) * 4
  * (bn*(bk+pad_b) for the second term when trans_b), the padded
  * counterpart of hint.smem_cost * pipeline_depth (src/roller.py:385); *threads (may be NULL)
  * receives 64 * (bm/wm) * (bn/wn). */
@@ -184,7 +186,7 @@ int rl_gemm_plans_clear(void);
  * src/roller.py:536 (the reference floors; ragged tiles are predicated here when cfg.edge).
  * Rejects, with RL_ERR_INVALID_ARG and before anything is launched, shapes the plan was not built
  * for: vec=4 with K, N or a leading dimension not a multiple of 4 or a base pointer not 16-byte
- * aligned; edge=0 with a dimension that its tile does not divide.  M==0 or N==0 is a no-op;
+ * aligned; edge=0 with a dimension that its tile does not divide; edge=2 with bk not dividing K.  M==0 or N==0 is a no-op;
  * K==0 writes zeros (or leaves C when accumulating). */
 int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
                         int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream);

@@ -266,8 +266,6 @@ class Policy:
     # registers per lane the MFMA kernel needs besides its accumulators and operand fragments:
     # addresses, loop state, buffer resources (measured: 40-60)
     REG_OVERHEAD = 50
-    # wave tiles of at most this many elements list the 16x16x4 variant first
-    SMALL_WAVE_TILE = 64 * 64
 
     def __init__(self, config: MatmulConfig, arch: TileDevice,
                  pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> None:
@@ -389,6 +387,10 @@ class Policy:
             s for s in self.get_reduce_step_candidates(self.matmul_config.K)
             if s % td.rstep == 0 and td.infer_smem_usage(s) <= limit
         ] or [td.rstep]
+        if self.arch.has_matrix_cores:
+            # a step that lets the loads go straight to LDS beats a longer one that does not
+            direct = [s for s in steps if loads_go_direct_to_lds(self.matmul_config, td.block_tile, s, self.pipeline_depth)]
+            steps = direct or steps
         td.rstep = max(steps, key=lambda s: self._coalesced_score(td.block_tile, s, "raw"))
         td.smem_cost = td.infer_smem_usage()
 
@@ -396,10 +398,18 @@ class Policy:
 
     def score_block_size(self, n: int):
         """(distance of the warp count from one warp per scheduler, fraction of idle lanes in
-        the last warp); smaller is better."""
+        the last warp); smaller is better.  On devices with matrix cores the imbalance between
+        the SIMDs comes first."""
         warp, part = self.arch.warp_size, self.arch.sm_partition * self.arch.waves_per_partition
         warps = -(-n // warp)
-        return (max(warps / part, part / warps), (warps * warp - n) / n)
+        score = (max(warps / part, part / warps), (warps * warp - n) / n)
+        if self.arch.has_matrix_cores:
+            # a wave count that is not a multiple of the SIMD count leaves matrix pipes idle while
+            # the fullest SIMD finishes (3 waves: one of four SIMDs idle; 5: one SIMD does double
+            # duty): that imbalance ranks before the distance from the target
+            simds = self.arch.sm_partition
+            score = (-(-warps // simds) * simds / warps,) + score
+        return score
 
     def recommend_block_size(self, td: TileDict) -> List[int]:
         """Thread counts worth trying for ``td``: divisors of the tile area up to 1024, best first."""
@@ -411,13 +421,14 @@ class Policy:
         Without matrix cores the first block size that cannot be tiled ends the sequence (the
         reference's behaviour).  With matrix cores such a block size is skipped -- most thread
         counts are not a whole number of waves or do not split into MFMA blocks -- and a block
-        size that works yields one copy per matrix-instruction shape that fits."""
+        size that works yields its wave tile with the matrix instruction the device model prefers
+        for that size (``_assign_wave_tiles`` lists the alternatives)."""
         for block_size in self.recommend_block_size(td):
             if self.arch.has_matrix_cores:
                 done = self._assign_wave_tiles(td, block_size)
                 if not done:
                     continue
-                yield from done
+                yield done[0]
             else:
                 one = self._assign_thread_tile(td, block_size)
                 if one is None:
@@ -486,10 +497,9 @@ class Policy:
             td.threads = block_size
             out.append(td.clone())
         # The instruction with the longer k (16x16x4) moves half as many accumulator bytes per FLOP,
-        # which leaves the register file free for LDS fragment reads: it wins on small wave tiles,
-        # where those reads are dense (measured 1-2 % on wave tiles up to 64x64); the larger
-        # instruction wins on large ones.
-        if len(out) > 1 and math.prod(out[0].wave_tile) <= self.SMALL_WAVE_TILE:
+        # which leaves the register file free for LDS fragment reads; up to the wave-tile size the
+        # device model names it is listed first.
+        if len(out) > 1 and math.prod(out[0].wave_tile) <= arch.long_k_mfma_up_to:
             out.sort(key=lambda t: t.mfma)
         return out
 

@@ -56,6 +56,8 @@ class TileDevice:
     # ``tile_fixed_seconds`` (pipeline fill) on top of storing its results
     mfma_efficiency: Tuple[float, float] = (1.0, 0.0)
     tile_fixed_seconds: float = 0.0
+    # wave tiles of at most this many elements list the matrix instruction with the longer k first
+    long_k_mfma_up_to: int = 0
 
     def get_avaliable_tensorintrin_shapes(self) -> List[Tuple[int, int, int]]:
         """Matrix-instruction shapes of the device (name kept from the reference, arch.py:36)."""
@@ -116,8 +118,10 @@ class MI355X(TileDevice):
     # the kernel's register-staged path pads every row of the LDS A tile by one 16-byte unit; its
     # direct-to-LDS path (K, N multiples of 4 and a power-of-two reduce step) swizzles instead
     lds_row_pad: int = 4
-    # two waves per SIMD let one wave's LDS traffic and barriers hide behind the other's MFMAs
-    waves_per_partition: int = 2
+    # waves per SIMD that the block-size recommendation tries first.  With loads going straight to
+    # LDS one wave per SIMD is enough to keep the matrix pipe fed, and its larger wave tile reads
+    # fewer operand bytes per FLOP (fitted to the committed sweep, see ``calibrate.py``)
+    waves_per_partition: int = 1
     # 256 architectural + 256 accumulation registers per lane, shared by the waves of a SIMD
     regs_per_lane: int = 512
     mfma_shapes: List[Tuple[int, int, int]] = field(default_factory=lambda: [(32, 32, 2), (16, 16, 4)])
@@ -126,8 +130,12 @@ class MI355X(TileDevice):
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
     # (a test refits it): about 0.95 for 256x256 tiles, 0.81 for 32x64
-    mfma_efficiency: Tuple[float, float] = (0.972, 3.456)
+    mfma_efficiency: Tuple[float, float] = (0.992, 2.73)
     tile_fixed_seconds: float = 1.0e-6
+    # 16x16x4 moves half as many accumulator bytes per FLOP as 32x32x2, which leaves the register
+    # file free for LDS fragment reads: it wins on every wave tile it fits (up to 64x128; a wave
+    # keeps at most 32 blocks), by 0.3-1 % in the committed sweep
+    long_k_mfma_up_to: int = 64 * 128
     smem_cap: int = field(init=False)
     max_smem_usage: int = field(init=False)
 

@@ -27,6 +27,7 @@ import pandas as pd
 from .analyze import DEFAULT_PIPELINE_DEPTH, MatmulConfig, get_roller_hints
 from .arch import MI355X, TileDevice
 from .roller import Compiler, run_baseline, run_eval, run_vendor_baseline
+from .tuner import DEFAULT_TOPK, TIE_MARGIN
 
 PIPELINE_DEPTH = DEFAULT_PIPELINE_DEPTH
 
@@ -39,7 +40,7 @@ README_SHAPES: List[Tuple[int, int, int]] = [
 ]
 
 
-def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
+def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = DEFAULT_TOPK,
               arch: Optional[TileDevice] = None, baseline: bool = True,
               csv_path: Optional[os.PathLike] = "benchmark_results.csv",
               dump_path: Optional[os.PathLike] = None, repeat_times: int = 20,
@@ -98,7 +99,9 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = 20,
                 compile_s += func.compile_ms / 1e3
                 t, gflops = run_eval(func, pipeline_depth, hint, repeat_times=repeat_times,
                                      seed=seed, distribution=distribution)
-                if t < best_time:
+                # the policy's order decides near ties: a later hint must win by more than the
+                # run-to-run spread of the measurement to displace an earlier one
+                if t < best_time * (1.0 - TIE_MARGIN):
                     best_time, best_gflops, best_hint, best_rank = t, gflops, hint, i + 1
                     best_info = dict(func.last_eval)
             except Exception as e:
@@ -213,7 +216,7 @@ def main(argv=None) -> None:
     ap = argparse.ArgumentParser(description="Roller fp32 GEMM sweep on MI355X")
     ap.add_argument("--shapes", default="readme", choices=["readme", "full"],
                     help="readme: M0..M13; full: all 27 products of {2048,4096,8192}")
-    ap.add_argument("--topk", type=int, default=20)
+    ap.add_argument("--topk", type=int, default=DEFAULT_TOPK, help="hints tried per shape (the reference tries 20)")
     ap.add_argument("--no-baseline", action="store_true")
     ap.add_argument("--csv", default="benchmark_results.csv")
     ap.add_argument("--dump", default=None, help="directory for kernel source / ISA dumps")

@@ -46,6 +46,9 @@ SHAPES.update({"cfg4": (3000, 5000, 1536), "1024x1024x1024": (1024, 1024, 1024),
                "1536x1536x1536": (1536, 1536, 1536), "1000x1000x1000": (1000, 1000, 1000)})
 
 
+MIN_FIT_MS = 0.1   # shortest measurement the efficiency fit uses
+
+
 def shape_of(name: str) -> Tuple[int, int, int]:
     if name in SHAPES:
         return SHAPES[name]
@@ -97,7 +100,8 @@ def best_per_block_tile(records: Iterable[dict]) -> List[dict]:
 def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
     """Least-squares ``efficiency = base - slope * (1/m + 1/n)`` over the best record of every
     (shape, block tile) whose tile grid fills at least three quarters of its last round of CUs
-    (a sparse last round measures the tail, not the tile).  Deterministic: closed-form normal
+    (a sparse last round measures the tail, not the tile) and that ran for at least ``MIN_FIT_MS``
+    (below that the launch itself is a visible share).  Deterministic: closed-form normal
     equations, records in sorted order."""
     arch = arch or MI355X()
     xs, ys = [], []
@@ -106,7 +110,7 @@ def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
         m, n = r["block_tile"]
         tiles = (-(-M // m)) * (-(-N // n))
         last_round = tiles % arch.compute_max_core or arch.compute_max_core
-        if M % m or N % n or last_round < 0.75 * arch.compute_max_core:
+        if M % m or N % n or last_round < 0.75 * arch.compute_max_core or r["ms"] < MIN_FIT_MS:
             continue
         eff = observed_efficiency(r, arch)
         if eff is None or not 0.3 < eff < 1.05:
@@ -123,6 +127,53 @@ def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
     resid = [y - (base + slope * x) for x, y in zip(xs, ys)]
     return {"mfma_efficiency": (round(base, 3), round(-slope, 2)), "base": base, "slope": -slope, "points": len(xs),
             "rms_residual": math.sqrt(math.fsum(e * e for e in resid) / n_pts)}
+
+
+def _geo_mean(ratios: Sequence[float]) -> float:
+    return math.exp(math.fsum(math.log(r) for r in ratios) / len(ratios))
+
+
+def fit_waves_per_simd(records: Sequence[dict], arch: Optional[TileDevice] = None, min_tile: int = 128 * 128) -> dict:
+    """Which block size the recommendation should try first: for every (shape, block tile) of at
+    least ``min_tile`` elements measured both with one and with two waves per SIMD, the ratio of
+    the two best times; the geometric mean over all pairs decides (``waves_per_partition``)."""
+    arch = arch or MI355X()
+    one, two = arch.warp_size * arch.sm_partition, 2 * arch.warp_size * arch.sm_partition
+    best: Dict[tuple, Dict[int, float]] = {}
+    for r in records:
+        if math.prod(r["block_tile"]) < min_tile or r["threads"] not in (one, two):
+            continue
+        slot = best.setdefault((tuple(r["shape"]), tuple(r["block_tile"])), {})
+        slot[r["threads"]] = min(slot.get(r["threads"], float("inf")), r["ms"])
+    ratios = [t[two] / t[one] for _, t in sorted(best.items()) if one in t and two in t]
+    if not ratios:
+        raise ValueError("no block tile was measured at both block sizes")
+    mean = _geo_mean(ratios)
+    return {"waves_per_partition": 1 if mean >= 1.0 else 2, "two_over_one": mean, "pairs": len(ratios)}
+
+
+def fit_long_k_mfma(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
+    """Up to which wave-tile size the instruction with the longer k (16x16x4) should be listed
+    first: for every wave-tile size, the geometric mean of time(32x32x2) / time(16x16x4) over the
+    (shape, block tile, wave tile) triples measured with both; the largest size whose mean is
+    above 1, with every smaller size above 1 as well (``long_k_mfma_up_to``)."""
+    by: Dict[tuple, Dict[int, float]] = {}
+    for r in records:
+        key = (tuple(r["shape"]), tuple(r["block_tile"]), tuple(r["wave_tile"]))
+        slot = by.setdefault(key, {})
+        slot[r["mfma"]] = min(slot.get(r["mfma"], float("inf")), r["ms"])
+    per_size: Dict[int, List[float]] = {}
+    for (_, _, wave_tile), t in sorted(by.items()):
+        if 16 in t and 32 in t:
+            per_size.setdefault(math.prod(wave_tile), []).append(t[32] / t[16])
+    means = {size: _geo_mean(v) for size, v in sorted(per_size.items())}
+    up_to = 0
+    for size, mean in means.items():
+        if mean <= 1.0:
+            break
+        up_to = size
+    return {"long_k_mfma_up_to": up_to, "mi32_over_mi16_by_wave_tile_elems": {k: round(v, 4) for k, v in means.items()},
+            "pairs": sum(len(v) for v in per_size.values())}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -169,6 +220,29 @@ def check(records: Sequence[dict], arch: Optional[TileDevice] = None, topk: int 
 # measuring (GPU)
 # ---------------------------------------------------------------------------------------------
 
+def candidate_hints(cfg: MatmulConfig, arch: TileDevice, topk: int, depth: int = DEFAULT_PIPELINE_DEPTH) -> List[TileDict]:
+    """What a calibration run times for one problem: the policy's block tiles in its current order
+    and, for each, the first two block sizes that split into wave tiles with EVERY matrix
+    instruction that fits -- also the alternatives the policy itself would not emit, because the
+    fits of the wave and instruction preferences need both sides of each comparison."""
+    policy = Policy(cfg, arch, depth)
+    out: List[TileDict] = []
+    for td in policy.get_block_tiles_candidates([1, 1], policy._assign_reduce_step()):
+        policy._expand_reduce_axis(td)
+        sizes = 0
+        for block_size in policy.recommend_block_size(td):
+            done = policy._assign_wave_tiles(td, block_size)
+            if not done:
+                continue
+            out.extend(done)
+            sizes += 1
+            if sizes == 2:
+                break
+        if len(out) >= topk:
+            break
+    return out[:topk]
+
+
 def measure(shape_names: Sequence[str], topk: int, depth: int = DEFAULT_PIPELINE_DEPTH, chunk: int = 8,
             say=lambda *a: print(*a, file=sys.stderr, flush=True)) -> dict:
     import numpy as np
@@ -190,9 +264,8 @@ def measure(shape_names: Sequence[str], topk: int, depth: int = DEFAULT_PIPELINE
         A, B = make_inputs(cfg, 0, "uniform")
         bufs = (DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray.zeros((M, N)))
         del A, B
-        hints = get_roller_hints(cfg, arch, topk=topk, pipeline_depth=depth)
         cands = []
-        for rank, hint in enumerate(hints, 1):
+        for rank, hint in enumerate(candidate_hints(cfg, arch, topk, depth), 1):
             try:
                 g = hint_to_gemm_config(cfg, hint, depth)
                 cands.append((rank, hint, g, GemmPlan(g)))
@@ -244,9 +317,15 @@ def main(argv=None) -> int:
     data = load(Path(args.data))
     if args.cmd == "fit":
         res = fit(data["records"])
-        now = MI355X().mfma_efficiency
+        now = MI355X()
         print(f"fitted mfma_efficiency = {res['mfma_efficiency']} from {res['points']} block tiles "
-              f"(rms residual {res['rms_residual']:.4f}); arch.MI355X has {tuple(now)}")
+              f"(rms residual {res['rms_residual']:.4f}); arch.MI355X has {tuple(now.mfma_efficiency)}")
+        waves = fit_waves_per_simd(data["records"])
+        print(f"fitted waves_per_partition = {waves['waves_per_partition']} (two waves per SIMD take {waves['two_over_one']:.4f} x "
+              f"the time of one, {waves['pairs']} block tiles); arch.MI355X has {now.waves_per_partition}")
+        instr = fit_long_k_mfma(data["records"])
+        print(f"fitted long_k_mfma_up_to = {instr['long_k_mfma_up_to']} (32x32x2 over 16x16x4 by wave-tile elements: "
+              f"{instr['mi32_over_mi16_by_wave_tile_elems']}); arch.MI355X has {now.long_k_mfma_up_to}")
         return 0
     rows = check(data["records"], topk=args.topk)
     for r in rows:

@@ -77,7 +77,7 @@ def profiled_bench(workload: str, counters: Optional[List[str]], work: Path, tag
     bench JSON line plus, per counter, the mean value over the kernel's dispatches."""
     bench_cmd = [sys.executable, str(BENCH), "--workload", workload, "--steps", str(steps), "--warmup", "1"]
     if workload != "copy":
-        bench_cmd.append("--no-cpu-baseline")
+        bench_cmd += ["--no-cpu-baseline", "--lean"]
     out_dir = work / tag
     cmd = bench_cmd
     if counters:

@@ -24,17 +24,20 @@
 //               global loads of step k+1 in flight during the MFMAs of step k; 3 = two LDS buffers
 //               plus a register stage: global loads run two steps ahead, and the LDS fragments of
 //               the next MFMA group are read while the current group executes, also across the
-//               barrier that ends a K step
+//               barrier that ends a K step; 4 and 5 (DIRECT only) = the same with three and four
+//               LDS buffers, so that loads run two and three K steps ahead of the MFMAs -- for
+//               short K steps whose MFMA time does not cover a trip to HBM
 //   PAD_A,PAD_B extra floats per LDS row of the A tile ([BM][BK+PAD_A]) and B tile ([BK][BN+PAD_B])
 //   VEC         4 = 128-bit global accesses (needs K%4==0, N%4==0, lda/ldb/ldc%4==0 and 16-byte
 //               aligned base pointers), 1 = dword accesses with per-element predicates
-//   EDGE        1 = predicate ragged tiles (any M, N, K), 0 = host guarantees BM|M, BN|N, BK|K
+//   EDGE        1 = predicate ragged tiles (any M, N, K), 2 = M and N may be ragged but the host
+//               guarantees BK|K (no per-step K predicates), 0 = host guarantees BM|M, BN|N, BK|K
 //   SWZ         workgroup-id remap: bit0 = give every XCD a contiguous run of tiles,
 //               bit1 = walk the tile grid in panels of GROUP tile rows
 //   GROUP, NXCD panel height in tiles; number of XCDs the dispatcher round-robins over
 //   ACCUM       1 = C += A*B (what linalg.matmul means, roller.py:62), 0 = C = A*B
 //   DIRECT      1 = global loads write LDS directly (buffer_load_dwordx4 ... lds), no staging
-//               registers and no LDS write instructions; needs STAGES=3, VEC=4, PAD_A=PAD_B=0
+//               registers and no LDS write instructions; needs STAGES>=3, VEC=4, PAD_A=PAD_B=0
 //               and BK a power of two.
 //               A wave's load lands as 64 consecutive 16-byte units, so rows cannot be padded;
 //               instead the 16-byte chunks of every A row are XOR-swizzled with the row number
@@ -54,10 +57,12 @@
 //     ds_read_b128; the four values feed four consecutive MFMAs.  MFMA t therefore contracts over
 //     k = kk + 4*g + t for lane group g (g = lane / MI), and the B operand of that MFMA is read
 //     from row kk + 4*g + t.
-//   * B stays N-contiguous in LDS.  A lane reads VN consecutive columns with one ds_read and the
-//     VN values feed VN different column blocks, so block bj of a wave owns the columns
-//     wn0 + (bj/VN)*MI*VN + VN*(lane%MI) + bj%VN.  In the epilogue the same VN accumulators are
-//     adjacent in memory again and leave as one vector store.
+//   * B stays N-contiguous in LDS.  A lane reads w consecutive columns with one ds_read and the
+//     w values feed w different column blocks.  The TN column blocks of a wave are cut into
+//     segments of w = 4 blocks, then one of 2 and one of 1 for what is left (TN = 8: 4+4; 5: 4+1;
+//     6: 4+2; 3: 2+1); a segment that starts at block b0 covers the MI*w columns from
+//     wn0 + b0*MI, and block b0+e owns the columns wn0 + b0*MI + w*(lane%MI) + e.  In the
+//     epilogue the same w accumulators are adjacent in memory again and leave as one vector store.
 // Rows of LDS-A are padded so that (BK+PAD_A)/4 is odd: the 16-byte reads of lanes in consecutive
 // rows then fall into distinct bank groups.
 //
@@ -123,6 +128,7 @@
 #define TRANS_B 0
 #endif
 
+#define EDGE_K (EDGE == 1) /* the K extent may be ragged as well */
 #define NWM (BM / WM)
 #define NWN (BN / WN)
 #define NWAVES (NWM * NWN)
@@ -131,10 +137,12 @@
 #define TN (WN / MI)
 #define KG (64 / MI)       /* lane groups along k inside one MFMA (= its k extent) */
 #define KSUPER (4 * KG)    /* k covered by the four MFMAs fed from one 128-bit A read */
-/* column blocks that one B read feeds: the widest of 4, 2, 1 that divides TN (TN = 3, 5: dword
- * reads; 6, 10: 64-bit reads; multiples of 4: 128-bit reads) */
-#define VN (TN % 4 == 0 ? 4 : (TN % 2 == 0 ? 2 : 1))
-#define NVB (TN / VN)
+/* segments of column blocks that one B read feeds: TN / 4 of four blocks (128-bit reads), then
+ * one of two (64-bit) and one of one (32-bit) for the remainder */
+#define NSEG4 (TN / 4)
+#define HAS_SEG2 ((TN % 4) / 2)
+#define HAS_SEG1 (TN % 2)
+#define NSEG (NSEG4 + HAS_SEG2 + HAS_SEG1)
 #define LDA_S (BK + PAD_A)
 #if TRANS_B
 #define LDB_S (BK + PAD_B)
@@ -145,7 +153,7 @@
 #endif
 #define A_STAGE (BM * LDA_S)
 #define STAGE_FLOATS (A_STAGE + B_STAGE)
-#define LDS_BUFS (STAGES >= 2 ? 2 : 1)
+#define LDS_BUFS (STAGES >= 3 ? STAGES - 1 : STAGES)
 #define SUPERS (BK / KSUPER) /* MFMA groups per K step, each fed by one round of fragment reads */
 #define A_UNITS (BM * BK / 4)
 #define B_UNITS (BK * BN / 4)
@@ -168,10 +176,24 @@ static_assert(TM * TN <= 32, "at most 32 MFMA blocks per wave: beyond that the a
 static_assert(BK % KSUPER == 0, "BK must be a multiple of 4*(64/MI)");
 static_assert(PAD_A % 4 == 0 && PAD_B % 4 == 0, "LDS rows stay 16-byte aligned");
 static_assert(TRANS_B == 0 || TRANS_B == 1, "TRANS_B is a flag");
+static_assert(EDGE >= 0 && EDGE <= 2, "EDGE: 0 none, 1 all three extents, 2 M and N only");
 static_assert(NT <= 1024, "at most 16 waves per workgroup");
-static_assert(STAGES >= 1 && STAGES <= 3, "pipeline depth 1, 2 or 3");
+static_assert(STAGES >= 1 && STAGES <= 5, "pipeline depth 1 to 5");
+static_assert(STAGES <= 3 || DIRECT, "more than two LDS buffers only with direct-to-LDS loads");
 static_assert(VEC == 4 || VEC == 1, "global access width");
-static_assert(!DIRECT || (STAGES == 3 && VEC == 4 && PAD_A == 0 && PAD_B == 0), "DIRECT needs STAGES=3, VEC=4, no padding");
+static_assert(!DIRECT || (STAGES >= 3 && VEC == 4 && PAD_A == 0 && PAD_B == 0), "DIRECT needs STAGES>=3, VEC=4, no padding");
+/* Waiting for "all but the newest n tiles" counts this wave's outstanding loads, which is exact
+ * only if every wave issues the same number of loads per tile. */
+#define LOADS_PER_TILE (A_PER_T + B_PER_T)
+#define EXACT_LOADS (A_UNITS % NT == 0 && B_UNITS % NT == 0)
+static_assert(LDS_BUFS <= 2 || EXACT_LOADS, "three or more LDS buffers need operand tiles that divide evenly over the threads");
+static_assert(LDS_BUFS <= 2 || (LDS_BUFS - 2) * LOADS_PER_TILE <= 63, "too many loads in flight for the 6-bit vmcnt");
+/* the prologue may start on tile 0 while the other requested tiles are still in flight, if that
+ * count can be waited for exactly; otherwise it waits for everything */
+#define PROLOGUE_IN_FLIGHT ((EXACT_LOADS && (LDS_BUFS - 1) * LOADS_PER_TILE <= 63) ? (LDS_BUFS - 1) * LOADS_PER_TILE : 0)
+/* s_waitcnt that waits until at most n vector-memory operations of this wave are outstanding
+ * (vmcnt is split over bits 3:0 and 15:14; expcnt and lgkmcnt are left at "do not wait") */
+#define WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 0xf) | ((((n) >> 4) & 0x3) << 14))
 static_assert(!DIRECT || (A_UNITS % 64 == 0 && B_UNITS % 64 == 0), "DIRECT moves whole waves of 16-byte units");
 static_assert(!DIRECT || (BK & (BK - 1)) == 0, "DIRECT swizzles A rows with XOR: BK must be a power of two");
 static_assert(LDS_BUFS * STAGE_FLOATS * 4 <= 160 * 1024, "tile does not fit the 160 KB LDS of a CU");
@@ -196,15 +218,11 @@ typedef v4f acc_t;
 #define ACC_ROW(r, g) (4 * (g) + (r))
 #endif
 
-#if VN == 4
-typedef v4f bvec_t;
-#elif VN == 2
-typedef v2f bvec_t;
-#else
-typedef float bvec_t;
-#endif
-
 #define DEV static __device__ __forceinline__
+
+// first block and width of B-read segment s
+DEV constexpr int seg_first(int s) { return s < NSEG4 ? 4 * s : (s == NSEG4 && HAS_SEG2 ? 4 * NSEG4 : TN - 1); }
+DEV constexpr int seg_width(int s) { return s < NSEG4 ? 4 : (s == NSEG4 && HAS_SEG2 ? 2 : 1); }
 
 template <int V>
 struct int_c {
@@ -256,11 +274,14 @@ DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool
 }
 
 #if TRANS_B
-// Column of the block tile that LDS row `row` of the Bt tile holds.  Block bj of a wave owns the
-// columns (bj/VN)*MI*VN + VN*lane + bj%VN of its wave tile; row bj*MI + lane holds that column.
+// Column of the block tile that LDS row `row` of the Bt tile holds.  Block bj = b0 + e of a wave,
+// in a segment of width sw that starts at block b0, owns the columns b0*MI + sw*lane + e of its
+// wave tile; row bj*MI + lane holds that column.
 DEV int bt_col_of_row(int row) {
-  const int w = row / WN, q = row % WN, v = q / (MI * VN), rem = q % (MI * VN);
-  return w * WN + v * MI * VN + VN * (rem % MI) + rem / MI;
+  const int w = row / WN, q = row % WN, bj = q / MI, lane = q % MI;
+  const int b0 = bj < 4 * NSEG4 ? (bj & ~3) : (HAS_SEG2 && bj < 4 * NSEG4 + 2 ? 4 * NSEG4 : TN - 1);
+  const int sw = bj < 4 * NSEG4 ? 4 : (HAS_SEG2 && bj < 4 * NSEG4 + 2 ? 2 : 1);
+  return w * WN + b0 * MI + sw * lane + (bj - b0);
 }
 #endif
 
@@ -405,7 +426,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < A_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (A_UNITS % NT == 0 || first < A_UNITS) {
-        const bool ok = a_ok[i] && (!EDGE || k0 + a_kcol[i] < K);
+        const bool ok = a_ok[i] && (!EDGE_K || k0 + a_kcol[i] < K);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr_t)(As + first * 4), 16, ok ? a_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -413,7 +434,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < B_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (B_UNITS % NT == 0 || first < B_UNITS) {
-        const bool ok = b_ok[i][0] && (!EDGE || k0 + b_krow[i] < K);  // K % 4 == 0: a chunk is in or out as a whole
+        const bool ok = b_ok[i][0] && (!EDGE_K || k0 + b_krow[i] < K);  // K % 4 == 0: a chunk is in or out as a whole
         __builtin_amdgcn_raw_ptr_buffer_load_lds(br, (lds_ptr_t)(Bs + first * 4), 16, ok ? b_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -432,18 +453,18 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < A_PER_T; ++i) {
       const int k = k0 + a_kcol[i];
       ra[i] = load_unit(ar, a_goff[i],
-                        a_ok[i] && (!EDGE || k + 0 < K), a_ok[i] && (!EDGE || k + 1 < K),
-                        a_ok[i] && (!EDGE || k + 2 < K), a_ok[i] && (!EDGE || k + 3 < K));
+                        a_ok[i] && (!EDGE_K || k + 0 < K), a_ok[i] && (!EDGE_K || k + 1 < K),
+                        a_ok[i] && (!EDGE_K || k + 2 < K), a_ok[i] && (!EDGE_K || k + 3 < K));
     }
 #pragma unroll
     for (int i = 0; i < B_PER_T; ++i) {
 #if TRANS_B
       const int k = k0 + b_krow[i];
       rb[i] = load_unit(br, b_goff[i],
-                        b_ok[i][0] && (!EDGE || k + 0 < K), b_ok[i][1] && (!EDGE || k + 1 < K),
-                        b_ok[i][2] && (!EDGE || k + 2 < K), b_ok[i][3] && (!EDGE || k + 3 < K));
+                        b_ok[i][0] && (!EDGE_K || k + 0 < K), b_ok[i][1] && (!EDGE_K || k + 1 < K),
+                        b_ok[i][2] && (!EDGE_K || k + 2 < K), b_ok[i][3] && (!EDGE_K || k + 3 < K));
 #else
-      const bool kin = !EDGE || k0 + b_krow[i] < K;
+      const bool kin = !EDGE_K || k0 + b_krow[i] < K;
       rb[i] = load_unit(br, b_goff[i], b_ok[i][0] && kin, b_ok[i][1] && kin, b_ok[i][2] && kin,
                         b_ok[i][3] && kin);
 #endif
@@ -483,18 +504,20 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #elif TRANS_B
   const int b_frag = (wn0 + lr) * LDB_S + 4 * lg;       // + bj*MI*LDB_S + kk
 #else
-  const int b_frag = (4 * lg) * LDB_S + wn0 + VN * lr;  // + (kk+t)*LDB_S + v*MI*VN
+  const int b_frag = (4 * lg) * LDB_S + wn0;            // + (kk+t)*LDB_S + b0*MI + w*lr per segment
 #endif
 
   // One round of LDS fragment reads: TM 128-bit reads of A (four consecutive k each) and, for each
-  // of the four k slots, NVB vector reads of B (TRANS_B: TN 128-bit reads, four consecutive k of
-  // one column each).  Feeds 4*TM*TN MFMAs.
+  // of the four k slots, one vector read of B per segment (TRANS_B: TN 128-bit reads, four
+  // consecutive k of one column each).  Feeds 4*TM*TN MFMAs.
   struct frag_t {
     v4f a[TM];
 #if TRANS_B
     v4f b[TN];
 #else
-    bvec_t b[4][NVB];
+    v4f b4[4][NSEG4 > 0 ? NSEG4 : 1];
+    v2f b2[4];
+    float b1[4];
 #endif
   };
   auto read_frags = [&](frag_t& f, int stage, int kk) {
@@ -514,9 +537,13 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int bj = 0; bj < TN; ++bj) f.b[bj] = *(const v4f*)&Bs[b_frag + bj * MI * LDB_S + kk];
 #else
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
+    for (int t = 0; t < 4; ++t) {
+      const float* row = &Bs[b_frag + (kk + t) * LDB_S];
 #pragma unroll
-      for (int v = 0; v < NVB; ++v) f.b[t][v] = *(const bvec_t*)&Bs[b_frag + (kk + t) * LDB_S + v * MI * VN];
+      for (int v = 0; v < NSEG4; ++v) f.b4[t][v] = *(const v4f*)&row[4 * v * MI + 4 * lr];
+      if constexpr (HAS_SEG2) f.b2[t] = *(const v2f*)&row[4 * NSEG4 * MI + 2 * lr];
+      if constexpr (HAS_SEG1) f.b1[t] = row[(TN - 1) * MI + lr];
+    }
 #endif
   };
   auto mfma_frags = [&](const frag_t& f, int t0 = 0, int t1 = 4) {
@@ -528,17 +555,15 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
         for (int bj = 0; bj < TN; ++bj) {
 #if TRANS_B
           const float bval = f.b[bj][t];
-#elif VN == 1
-          const float bval = f.b[t][bj];
 #else
-          const float bval = f.b[t][bj / VN][bj % VN];
+          const float bval = bj < 4 * NSEG4 ? f.b4[t][bj / 4][bj % 4] : (HAS_SEG2 && bj < 4 * NSEG4 + 2 ? f.b2[t][bj - 4 * NSEG4] : f.b1[t]);
 #endif
           acc[bi][bj] = MFMA(f.a[bi][t], bval, acc[bi][bj]);
         }
   };
 
   // ---- main loop ----
-#if STAGES == 3
+#if STAGES >= 3
   if (KT > 0) {
     // Software pipeline.  At the top of step kt: tile kt is in LDS buffer kt&1, its first fragment
     // round is already in registers, and the staging registers hold tile kt+1 (loaded during step
@@ -548,9 +573,10 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // round of tile kt+1 is read -- so that the last MFMA group covers that read's latency.
     frag_t fr[2];
 #if DIRECT
-    fetch_direct(0, 0);
-    fetch_direct(1, 1);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of both tiles is in LDS
+#pragma unroll
+    for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(i, i);
+    // this wave's part of tile 0 is in LDS (of every requested tile when the loads per wave differ)
+    WAIT_VMCNT(PROLOGUE_IN_FLIGHT);
 #else
     fetch(0);
     stash(0);
@@ -562,11 +588,11 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // P = which of the two fragment sets holds round 0 of this step (compile-time, so that the
     // sets stay in fixed registers); the set alternates every round.
     // MFMAs and fragment reads per round; LDS writes and global loads per K step
-    constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NVB), W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
+    constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NSEG), W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
 
     auto step = [&](auto parity, int kt) {
       constexpr int P = decltype(parity)::value;
-      const int cur = kt & 1;
+      const int cur = (unsigned)kt % LDS_BUFS, nxt = (unsigned)(kt + 1) % LDS_BUFS;
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
@@ -578,16 +604,17 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       // loads of tile kt+2 behind every second MFMA instead of every one: measured 0.3-0.8 % faster)
 #if DIRECT
       mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 1);
-      // Tile kt+1 was requested one step ago, straight into the other buffer; once every wave's
-      // part has landed and all have met, buffer `cur` is free again and takes tile kt+2.
+      // Tile kt+1 was requested LDS_BUFS-1 steps ago, straight into the next buffer; once every
+      // wave's part has landed (the requests for later tiles may still be in flight) and all have
+      // met, buffer `cur` is free again and takes tile kt+LDS_BUFS.
 #if SCHED
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
 #endif
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      WAIT_VMCNT((LDS_BUFS - 2) * LOADS_PER_TILE);
       __syncthreads();
-      read_frags(fr[(P + SUPERS) & 1], cur ^ 1, 0);
-      fetch_direct(kt + 2, cur);
+      read_frags(fr[(P + SUPERS) & 1], nxt, 0);
+      fetch_direct(kt + LDS_BUFS, cur);
       mfma_frags(fr[(P + SUPERS - 1) & 1], 1, 4);
 #if SCHED
       {
@@ -602,7 +629,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
 #else
       mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
-      stash(cur ^ 1);
+      stash(nxt);
       fetch(kt + 2);
 #if SCHED
 #pragma unroll
@@ -611,7 +638,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       interleave_with_mfma<G / 2 - G / 4, L, 0x020>();
 #endif
       __syncthreads();
-      read_frags(fr[(P + SUPERS) & 1], cur ^ 1, 0);
+      read_frags(fr[(P + SUPERS) & 1], nxt, 0);
       mfma_frags(fr[(P + SUPERS - 1) & 1], 2, 4);
 #if SCHED
       interleave_with_mfma<G / 2, R, 0x100>();
@@ -620,7 +647,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     };
     auto last_step = [&](auto parity, int kt) {
       constexpr int P = decltype(parity)::value;
-      const int cur = kt & 1;
+      const int cur = (unsigned)kt % LDS_BUFS;
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
@@ -632,7 +659,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
 #endif
 #if DIRECT
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // the (empty) request for the tile past the end has drained
+      WAIT_VMCNT(0);  // the (empty) requests for the tiles past the end have drained
 #endif
     };
 
@@ -697,37 +724,38 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       const int row = wm0 + bi * MI + ACC_ROW(r, lg);
       const bool rok = !EDGE || m0 + row < M;
 #pragma unroll
-      for (int v = 0; v < NVB; ++v) {
-        const int col = wn0 + v * MI * VN + VN * lr;
+      for (int sg = 0; sg < NSEG; ++sg) {
+        const int b0 = seg_first(sg), sw = seg_width(sg);
+        const int col = wn0 + b0 * MI + sw * lr;
         const unsigned off = (unsigned)(row * ldc + col) * 4u;
-        float o[VN];
+        float o[4];
 #pragma unroll
-        for (int e = 0; e < VN; ++e) o[e] = acc[bi][v * VN + e][r];
-#if VEC == 4 && VN == 4
-        const unsigned po = rok && (!EDGE || n0 + col < N) ? off : OOB_OFFSET;
-        v4f out = {o[0], o[1], o[2], o[3]};
+        for (int e = 0; e < 4; ++e) o[e] = e < sw ? acc[bi][b0 + (e < sw ? e : 0)][r] : 0.0f;
+        if (VEC == 4 && sw == 4) {
+          const unsigned po = rok && (!EDGE || n0 + col < N) ? off : OOB_OFFSET;
+          v4f out = {o[0], o[1], o[2], o[3]};
 #if ACCUM
-        out += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(cr, po, 0, 0));
+          out += __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(cr, po, 0, 0));
 #endif
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, out), cr, po, 0, 0);
-#elif VEC == 4 && VN == 2
-        const unsigned po = rok && (!EDGE || n0 + col < N) ? off : OOB_OFFSET;
-        v2f out = {o[0], o[1]};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, out), cr, po, 0, 0);
+        } else if (VEC == 4 && sw == 2) {
+          const unsigned po = rok && (!EDGE || n0 + col < N) ? off : OOB_OFFSET;
+          v2f out = {o[0], o[1]};
 #if ACCUM
-        out += __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(cr, po, 0, 0));
+          out += __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(cr, po, 0, 0));
 #endif
-        __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, out), cr, po, 0, 0);
-#else
+          __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(v2u, out), cr, po, 0, 0);
+        } else {
 #pragma unroll
-        for (int e = 0; e < VN; ++e) {
-          const unsigned po = rok && (!EDGE || n0 + col + e < N) ? off + 4u * e : OOB_OFFSET;
-          float out = o[e];
+          for (int e = 0; e < sw; ++e) {
+            const unsigned po = rok && (!EDGE || n0 + col + e < N) ? off + 4u * e : OOB_OFFSET;
+            float out = o[e];
 #if ACCUM
-          out += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, po, 0, 0));
+            out += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(cr, po, 0, 0));
 #endif
-          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), cr, po, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), cr, po, 0, 0);
+          }
         }
-#endif
       }
     }
 }

@@ -122,15 +122,16 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
   if (c.bk % ksuper) return fail(RL_ERR_INVALID_ARG, "bk must be a multiple of %d for mi=%d, got %d", ksuper, c.mi, c.bk);
   if (c.pad_a < 0 || c.pad_b < 0 || c.pad_a % 4 || c.pad_b % 4)
     return fail(RL_ERR_INVALID_ARG, "pad_a/pad_b must be non-negative multiples of 4");
-  if (c.stages < 1 || c.stages > 3) return fail(RL_ERR_INVALID_ARG, "stages must be 1, 2 or 3, got %d", c.stages);
+  if (c.stages < 1 || c.stages > 5) return fail(RL_ERR_INVALID_ARG, "stages must be 1 to 5, got %d", c.stages);
   if (c.vec != 4 && c.vec != 1) return fail(RL_ERR_INVALID_ARG, "vec must be 4 or 1, got %d", c.vec);
-  if ((c.edge | 1) != 1 || (c.accum | 1) != 1) return fail(RL_ERR_INVALID_ARG, "edge and accum are 0 or 1");
+  if (c.edge < 0 || c.edge > 2) return fail(RL_ERR_INVALID_ARG, "edge is 0, 1 or 2, got %d", c.edge);
+  if ((c.accum | 1) != 1) return fail(RL_ERR_INVALID_ARG, "accum is 0 or 1");
   if (c.swz < 0 || c.swz > 3) return fail(RL_ERR_INVALID_ARG, "swz is a 2-bit mask");
   if ((c.swz & 2) && c.group <= 0) return fail(RL_ERR_INVALID_ARG, "group must be positive");
   if ((c.direct | 1) != 1) return fail(RL_ERR_INVALID_ARG, "direct is 0 or 1");
   if (c.direct) {
-    if (c.stages != 3 || c.vec != 4 || c.pad_a || c.pad_b)
-      return fail(RL_ERR_INVALID_ARG, "direct=1 needs stages=3, vec=4, pad_a=0, pad_b=0");
+    if (c.stages < 3 || c.vec != 4 || c.pad_a || c.pad_b)
+      return fail(RL_ERR_INVALID_ARG, "direct=1 needs stages>=3, vec=4, pad_a=0, pad_b=0");
     if (c.bk & (c.bk - 1)) return fail(RL_ERR_INVALID_ARG, "direct=1 needs bk to be a power of two (XOR swizzle), got %d", c.bk);
     if ((c.bm * c.bk / 4) % 64 || (c.bk * c.bn / 4) % 64)
       return fail(RL_ERR_INVALID_ARG, "direct=1 needs bm*bk and bk*bn to be multiples of 256 (whole waves of 16-byte units)");
@@ -138,7 +139,16 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
   if ((c.trans_b | 1) != 1) return fail(RL_ERR_INVALID_ARG, "trans_b is 0 or 1");
   const int nt = 64 * (c.bm / c.wm) * (c.bn / c.wn);
   if (nt > 1024) return fail(RL_ERR_INVALID_ARG, "%d threads per workgroup exceed 1024", nt);
-  const long lds = (long)(c.stages >= 2 ? 2 : 1) * ((long)c.bm * (c.bk + c.pad_a) + (c.trans_b ? (long)c.bn * (c.bk + c.pad_b) : (long)c.bk * (c.bn + c.pad_b))) * 4;
+  const int bufs = c.stages >= 3 ? c.stages - 1 : c.stages;  // LDS buffers: 1, 2, 2, 3, 4
+  if (c.stages > 3) {
+    if (!c.direct) return fail(RL_ERR_INVALID_ARG, "stages=%d (more than two LDS buffers) needs direct=1", c.stages);
+    const int a_units = c.bm * c.bk / 4, b_units = c.bk * c.bn / 4;
+    if (a_units % nt || b_units % nt)
+      return fail(RL_ERR_INVALID_ARG, "stages=%d needs bm*bk/4 and bk*bn/4 to be multiples of the %d threads", c.stages, nt);
+    if ((bufs - 2) * (a_units / nt + b_units / nt) > 63)
+      return fail(RL_ERR_INVALID_ARG, "stages=%d keeps %d loads per thread in flight; at most 63", c.stages, (bufs - 2) * (a_units / nt + b_units / nt));
+  }
+  const long lds = (long)bufs * ((long)c.bm * (c.bk + c.pad_a) + (c.trans_b ? (long)c.bn * (c.bk + c.pad_b) : (long)c.bk * (c.bn + c.pad_b))) * 4;
   if (lds > 160 * 1024) return fail(RL_ERR_INVALID_ARG, "%ld bytes of LDS exceed the 160 KB of a CU", lds);
   if (lds_bytes) *lds_bytes = (int)lds;
   if (threads) *threads = nt;
@@ -763,6 +773,8 @@ int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B
   }
   if (!c.edge && (M % c.bm || N % c.bn || K % c.bk))
     return fail(RL_ERR_INVALID_ARG, "edge=0 kernel needs bm|M, bn|N, bk|K (tile %dx%dx%d, problem %dx%dx%d)", c.bm, c.bn, c.bk, M, N, K);
+  if (c.edge == 2 && K % c.bk)
+    return fail(RL_ERR_INVALID_ARG, "edge=2 kernel needs bk|K (bk=%d, K=%d)", c.bk, K);
   // In-tile byte offsets are 32-bit inside the kernel; 0x80000000 is reserved as "out of range".
   const long lim = 0x7fffffffL;
   if ((long)c.bm * lda * 4 + (long)c.bk * 4 > lim || (c.trans_b ? (long)c.bn * ldb * 4 + (long)c.bk * 4 : (long)c.bk * ldb * 4 + (long)c.bn * 4) > lim ||

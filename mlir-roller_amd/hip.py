@@ -95,12 +95,19 @@ class GemmConfig:
     @property
     def lds_bytes(self) -> int:
         b_tile = self.bn * (self.bk + self.pad_b) if self.trans_b else self.bk * (self.bn + self.pad_b)
-        return min(self.stages, 2) * (self.bm * (self.bk + self.pad_a) + b_tile) * 4
+        return self.lds_buffers * (self.bm * (self.bk + self.pad_a) + b_tile) * 4
+
+    @property
+    def lds_buffers(self) -> int:
+        """LDS buffers per pipeline depth: 1, 2, 2 (plus a register stage), 3, 4."""
+        return self.stages - 1 if self.stages >= 3 else self.stages
 
     def tag(self) -> str:
         return (f"b{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_mi{self.mi}_s{self.stages}"
                 f"_p{self.pad_a}.{self.pad_b}_v{self.vec}_e{self.edge}_z{self.swz}.{self.group}"
                 f"_a{self.accum}" + ("_d1" if self.direct else "") + ("_tb" if self.trans_b else ""))
+
+    MAX_STAGES = 5
 
 
 # --------------------------------------------------------------------------------------------

@@ -61,8 +61,19 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
                              f"for {threads} threads and reduce step {bk}")
         (wm, wn), mi = split
     M, N, K = config.M, config.N, config.K
-    stages = max(1, min(3, int(pipeline_depth)))
+    stages = max(1, min(GemmConfig.MAX_STAGES, int(pipeline_depth)))
     vec = 4 if (K % 4 == 0 and N % 4 == 0) else 1
+    # Depths 4 and 5 (three and four LDS buffers) exist on the direct-to-LDS path only, for tiles
+    # that divide evenly over the threads and fit the CU's LDS; otherwise the deepest depth that
+    # does fit is taken.
+    threads = 64 * (bm // wm) * (bn // wn)
+    while stages > 3:
+        loads = (bm * bk // 4) // threads + (bk * bn // 4) // threads
+        if (loads_go_direct_to_lds(config, (bm, bn), bk, stages) and (bm * bk // 4) % threads == 0
+                and (bk * bn // 4) % threads == 0 and (stages - 3) * loads <= 63
+                and (stages - 1) * (bm * bk + bk * bn) * 4 <= MI355X().lds_bytes):
+            break
+        stages -= 1
     # At full depth and width the global loads go straight to LDS (swizzled A rows, no padding)
     # whenever both operand tiles are whole waves of 16-byte units and the K step is a power of
     # two (the swizzle is an XOR).
@@ -74,14 +85,16 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
     # Padding is an optimisation, fitting the CU is not: a hint whose policy ran for another depth
     # or layout may leave no room for it.
     lds_cap = MI355X().lds_bytes
-    footprint = lambda pa, pb: min(stages, 2) * (bm * (bk + pa) + (bn * (bk + pb) if trans_b else bk * (bn + pb))) * 4
+    buffers = stages - 1 if stages >= 3 else stages
+    footprint = lambda pa, pb: buffers * (bm * (bk + pa) + (bn * (bk + pb) if trans_b else bk * (bn + pb))) * 4
     if pad_b and footprint(pad_a, pad_b) > lds_cap:
         pad_b = 0
     if pad_a and footprint(pad_a, pad_b) > lds_cap:
         pad_a = 0
     return GemmConfig(
         bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi, stages=stages, pad_a=pad_a, pad_b=pad_b, vec=vec,
-        edge=0 if (M % bm == 0 and N % bn == 0 and K % bk == 0) else 1,
+        # 0: every extent is a whole number of tiles; 2: only M or N is ragged; 1: K is ragged too
+        edge=(0 if (M % bm == 0 and N % bn == 0) else 2) if K % bk == 0 else 1,
         swz=3, group=8, accum=1 if accumulate else 0, direct=direct, trans_b=1 if trans_b else 0,
     )
 

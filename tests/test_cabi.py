@@ -71,15 +71,19 @@ def test_config_check_accepts_and_sizes(hip_lib):
     (dict(mi=8), "mi must be"),
     (dict(wm=48), "does not divide block tile"),
     (dict(wm=64, wn=64, bm=64, bn=64, mi=32, bk=12), "bk must be a multiple"),
-    (dict(stages=4), "stages must be"),
+    (dict(stages=6), "stages must be"),
+    (dict(stages=4), "needs direct=1"),
+    (dict(stages=4, direct=1, pad_a=0, bm=32, bn=64, wm=32, wn=32, bk=8), "multiples of the 128 threads"),
+    (dict(stages=5, direct=1, pad_a=0, bm=256, bn=256, wm=128, wn=128, bk=32), "exceed the 160 KB"),
     (dict(vec=2), "vec must be"),
     (dict(pad_a=2), "pad_a/pad_b"),
     (dict(bm=512, bn=512, wm=128, wn=128, bk=64), "exceed"),
     (dict(bm=1024, bn=1024, wm=32, wn=32, bk=8), "threads per workgroup"),
-    (dict(edge=2), "edge and accum"),
+    (dict(edge=3), "edge is 0, 1 or 2"),
+    (dict(accum=2), "accum is 0 or 1"),
     (dict(mi=16, bk=8), "bk must be a multiple of 16"),
-    (dict(direct=1), "direct=1 needs stages=3"),
-    (dict(direct=1, stages=3, pad_a=0, vec=1), "direct=1 needs stages=3"),
+    (dict(direct=1), "direct=1 needs stages>=3"),
+    (dict(direct=1, stages=3, pad_a=0, vec=1), "direct=1 needs stages>=3"),
     (dict(direct=2), "direct is 0 or 1"),
     (dict(direct=1, stages=3, pad_a=0, bk=24), "power of two"),
 ])

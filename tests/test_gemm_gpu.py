@@ -133,6 +133,20 @@ CASES += [
     (GemmConfig(96, 192, 16, 48, 96, 16, 2, 4, 4, 4, 1, 3, 8, 0, 0, 1), [(200, 400, 48)]),                                 # transposed, 6 blocks, staged
     (GemmConfig(96, 96, 16, 48, 48, 16, 3, 4, 4, 1, 1, 3, 8, 0, 0, 1), [(101, 99, 37)]),                                   # transposed, 3 blocks, dword
 ]
+# edge=2 (M and N ragged, K a whole number of steps: no K predicates in the loop) and pipeline depths 4 and 5
+# (three and four LDS buffers, loads two and three K steps ahead): 1, 2, 3 and many K steps, fewer steps than buffers
+CASES += [
+    (GemmConfig(128, 128, 32, 64, 64, 32, 3, 0, 0, 4, 2, 3, 8, 0, 1), [(200, 300, 32), (130, 260, 96), (1, 4, 64)]),
+    (GemmConfig(192, 320, 32, 96, 160, 32, 3, 0, 0, 4, 2, 3, 8, 0, 1), [(400, 700, 96)]),
+    (GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 2), [(200, 300, 80)]),
+    (GemmConfig(128, 128, 16, 64, 64, 16, 3, 4, 4, 1, 2, 3, 8, 0, 0, 1), [(37, 53, 32)]),
+    (GemmConfig(128, 128, 32, 64, 64, 16, 4, 0, 0, 4, 0, 3, 8, 0, 1), [(256, 384, 32), (256, 384, 64), (256, 384, 96), (256, 384, 512)]),
+    (GemmConfig(128, 128, 32, 64, 64, 16, 5, 0, 0, 4, 1, 3, 8, 0, 1), [(200, 300, 32), (200, 300, 64), (200, 300, 96), (200, 300, 128), (200, 300, 200), (130, 260, 1000)]),
+    (GemmConfig(64, 64, 64, 16, 32, 16, 5, 0, 0, 4, 2, 3, 8, 0, 1), [(200, 300, 64), (200, 300, 448)]),
+    (GemmConfig(128, 128, 8, 64, 64, 32, 4, 0, 0, 4, 1, 3, 8, 0, 1), [(140, 132, 8), (140, 132, 24), (140, 132, 100)]),     # odd number of rounds per step
+    (GemmConfig(256, 256, 16, 128, 128, 32, 4, 0, 0, 4, 0, 3, 8, 0, 1), [(512, 512, 160)]),
+    (GemmConfig(128, 128, 32, 32, 64, 32, 4, 0, 0, 4, 1, 3, 8, 0, 1, 1), [(200, 300, 200)]),                                 # transposed operand
+]
 FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
 
 
@@ -455,20 +469,35 @@ def test_named_configs_full_size_through_policy_and_compiler(device, name, shape
     assert (tmp_path / "kernel.hip").exists() and (tmp_path / "kernel.json").exists()
 
 
-def test_m0_to_m13_exact_on_integer_inputs_at_full_size(device):
-    """Size-independent property: with inputs in {0..9} every partial sum is an integer below
-    2^24, so any correct summation order gives the same float32 bits as the host GEMM."""
+TUNER_TOPK = 8   # at least what the tuner tries by default, with room for a user's --topk 8
+
+
+def test_every_kernel_the_tuner_can_pick_is_exact_at_full_size(device):
+    """M0..M13 and the ragged 3000x5000x1536, every one of the policy's first hints (all the
+    tuner may time and keep), through ``Compiler`` at the sweep's pipeline depth.  Size-independent
+    property: with inputs in {0..9} every partial sum is an integer below 2^24, so any correct
+    summation order gives the same float32 bits as the host GEMM -- a wrong kernel can never be
+    timed, whatever rank it has."""
+    from mlir_roller_amd import tuner
+    assert TUNER_TOPK >= tuner.DEFAULT_TOPK
     arch = MI355X.from_device(device)
-    for i, shape in enumerate(bm.README_SHAPES):
+    launches = 0
+    for i, shape in enumerate(list(bm.README_SHAPES) + [(3000, 5000, 1536)]):
         cfg = MatmulConfig(*shape, 32)
-        hint = get_roller_hints(cfg, arch, topk=1)[0]
-        say(f"M{i}", shape, hint.block_tile, hint.wave_tile, hint.rstep)
+        hints = get_roller_hints(cfg, arch, topk=TUNER_TOPK, pipeline_depth=bm.PIPELINE_DEPTH)
+        assert len(hints) == TUNER_TOPK
         A, B = go.make_inputs(*shape, seed=i, distribution="integer")
-        func = roller.Compiler(cfg, hint, bm.PIPELINE_DEPTH).compile()
+        want = go.gemm_f32(A, B)
         dA, dB, dC = DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray((shape[0], shape[1]))
-        func(func.grid_dims(), func.block_dims(), (dA, dB, dC))
-        hip.synchronize()
-        assert np.array_equal(dC.get(), go.gemm_f32(A, B)), shape
+        for rank, hint in enumerate(hints, 1):
+            say(f"shape {i}", shape, "rank", rank, hint.block_tile, hint.wave_tile, hint.mfma, hint.rstep)
+            func = roller.Compiler(cfg, hint, bm.PIPELINE_DEPTH).compile()
+            dC.fill_bytes(0xFF)
+            func(func.grid_dims(), func.block_dims(), (dA, dB, dC))
+            hip.synchronize()
+            assert np.array_equal(dC.get(), want), (shape, rank, func.gemm_config.tag())
+            launches += 1
+    assert launches == 15 * TUNER_TOPK
 
 
 def small_integer_matrix(rows, cols, seed):

@@ -41,7 +41,7 @@ def test_direct_path_needs_a_power_of_two_k_step():
 def test_hint_to_gemm_config_ragged_problem():
     cfg = MatmulConfig(3000, 5000, 1536, 32)
     g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0])
-    assert g.edge == 1 and g.vec == 4                # 5000 and 1536 are multiples of 4
+    assert g.edge == 2 and g.vec == 4 and 1536 % g.bk == 0   # 5000 and 1536 are multiples of 4; K is a whole number of steps
     cfg = MatmulConfig(37, 53, 29, 32)
     g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0], pipeline_depth=3)
     assert g.edge == 1 and g.vec == 1 and g.direct == 0 and g.pad_a == 4   # dword path keeps padded rows
@@ -257,3 +257,32 @@ def test_kernel_arguments_are_typed_by_type_not_by_value():
         hip._pack_arg("x")
     with pytest.raises(ValueError):
         hip.Ptr(-1)
+
+
+def test_tuner_keeps_the_policys_order_on_near_ties():
+    from mlir_roller_amd import tuner
+    assert tuner.DEFAULT_TOPK <= 4                                                 # the reference tries 20
+    assert tuner.choose([(1, 1.000), (2, 0.997), (3, 0.996)]) == 1                 # within the spread: rank 1 stays
+    assert tuner.choose([(1, 1.000), (2, 0.990), (3, 0.989)]) == 2                 # 1 % faster displaces; 0.1 % more does not
+    assert tuner.choose([(3, 0.90), (1, 1.0), (2, 0.97)]) == 3                     # order of the list does not matter
+    assert tuner.choose([(1, 1.0), (2, 0.97), (3, 0.90)]) == 3
+    assert tuner.choose([(1, float("nan")), (2, 2.0), (3, float("inf")), (4, 0.0)]) == 2   # unusable timings are skipped
+    assert tuner.choose([]) == -1 and tuner.choose([(1, float("nan"))]) == -1
+    assert tuner.choose([(1, 1.0), (2, 0.996)], margin=0.0) == 2                   # margin 0: plain fastest
+    s = tuner.summarise([(1, 1.0), (2, 0.997), (3, 0.996)], 1)
+    assert s == {"kept_rank": 1, "fastest_rank": 3, "kept_over_fastest": 1.004, "top1_over_fastest": 1.004}
+    assert tuner.ramp_launches((2048, 2048, 2048)) >= 250 and tuner.ramp_launches((8192, 8192, 8192), 3) >= 5
+
+
+def test_sweep_applies_the_tie_rule(monkeypatch, tmp_path):
+    # three hints, the third 0.3 % faster than the first: the first is reported
+    times = iter([1.000, 1.002, 0.997])
+
+    class Fake:
+        compile_ms = 0.0
+        last_eval = {}
+
+    monkeypatch.setattr(bm, "Compiler", lambda *a, **k: type("C", (), {"compile": lambda self: Fake()})())
+    monkeypatch.setattr(bm, "run_eval", lambda *a, **k: (next(times), 1.0))
+    df = bm.benchmark([(2048, 2048, 2048)], topk=3, baseline=False, csv_path=None)
+    assert int(df["Best Hint Rank"][0]) == 1 and float(df["Roller Time (ms)"][0]) == 1.000

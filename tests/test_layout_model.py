@@ -26,7 +26,27 @@ def test_model_constants_are_the_templates():
     assert re.search(r"#define SWZ_N \(CPR >= 16 \? 16 : CPR\)", TEMPLATE)
     assert "(u % CPR) ^ ((row / RPL) % SWZ_N)" in TEMPLATE                       # writer side
     assert "((r * (KSUPER / 4) + lg) ^ ((lr / RPL) % SWZ_N)) * 4" in TEMPLATE      # reader side
-    assert "w * WN + v * MI * VN + VN * (rem % MI) + rem / MI" in TEMPLATE         # Bt row -> column
+    assert "return w * WN + b0 * MI + sw * lane + (bj - b0);" in TEMPLATE          # Bt row -> column
+    assert "#define NSEG4 (TN / 4)" in TEMPLATE and "#define HAS_SEG2 ((TN % 4) / 2)" in TEMPLATE and "#define HAS_SEG1 (TN % 2)" in TEMPLATE
+
+
+def segments(tn):
+    """(first block, width) of the B-read segments of a wave with ``tn`` column blocks: as many of
+    four blocks as fit, then one of two and one of one (``seg_first`` / ``seg_width`` of the template)."""
+    out = [(4 * s, 4) for s in range(tn // 4)]
+    if (tn % 4) // 2:
+        out.append((4 * (tn // 4), 2))
+    if tn % 2:
+        out.append((tn - 1, 1))
+    return out
+
+
+def test_segments_cover_the_column_blocks():
+    assert segments(8) == [(0, 4), (4, 4)] and segments(5) == [(0, 4), (4, 1)] and segments(6) == [(0, 4), (4, 2)]
+    assert segments(3) == [(0, 2), (2, 1)] and segments(7) == [(0, 4), (4, 2), (6, 1)] and segments(1) == [(0, 1)] and segments(2) == [(0, 2)]
+    for tn in range(1, 33):
+        blocks = [b0 + e for b0, w in segments(tn) for e in range(w)]
+        assert blocks == list(range(tn))
 
 
 @pytest.mark.parametrize("bk,mi,rows", [(8, 32, 128), (16, 32, 128), (32, 32, 256), (64, 32, 128), (128, 32, 64),
@@ -75,49 +95,61 @@ def test_padded_rows_of_the_staged_path_are_free_of_bank_conflicts(bk, pad, mi):
         assert len(groups) == 16
 
 
-@pytest.mark.parametrize("wn,mi,waves_n", [(32, 32, 4), (64, 32, 2), (128, 32, 2), (256, 32, 1), (16, 16, 4), (32, 16, 2), (64, 16, 2), (128, 16, 1)])
+WAVE_WIDTHS = [(32, 32), (64, 32), (128, 32), (256, 32), (16, 16), (32, 16), (64, 16), (128, 16),
+               (96, 32), (160, 32), (48, 16), (80, 16), (96, 16), (112, 16), (160, 16)]      # 3, 5, 6, 7, 10 column blocks too
+
+
+def epilogue_column(bj, lane, mi, tn):
+    """Column (inside the wave tile) to which the epilogue stores block bj's accumulator of ``lane``."""
+    b0, w = next(sg for sg in segments(tn) if sg[0] <= bj < sg[0] + sg[1])
+    return b0 * mi + w * lane + (bj - b0)
+
+
+@pytest.mark.parametrize("wn,mi,waves_n", [(wn, mi, 2) for wn, mi in WAVE_WIDTHS])
 def test_transposed_operand_rows_are_a_permutation_that_matches_the_epilogue(wn, mi, waves_n):
     tn = wn // mi
-    vn = 4 if tn >= 4 else tn
     bn = wn * waves_n
 
-    def col_of_row(row):
+    def col_of_row(row):                             # bt_col_of_row of the template
         w, q = divmod(row, wn)
-        v, rem = divmod(q, mi * vn)
-        return w * wn + v * mi * vn + vn * (rem % mi) + rem // mi
+        bj, lane = divmod(q, mi)
+        b0 = (bj & ~3) if bj < 4 * (tn // 4) else (4 * (tn // 4) if (tn % 4) // 2 and bj < 4 * (tn // 4) + 2 else tn - 1)
+        sw = 4 if bj < 4 * (tn // 4) else (2 if (tn % 4) // 2 and bj < 4 * (tn // 4) + 2 else 1)
+        return w * wn + b0 * mi + sw * lane + (bj - b0)
 
     assert sorted(col_of_row(r) for r in range(bn)) == list(range(bn))
     # block bj of wave w reads LDS row w*wn + bj*mi + lane; the epilogue stores that accumulator to
-    # column w*wn + (bj // vn)*mi*vn + vn*lane + bj % vn
+    # the column its segment assigns
     for w, bj, lane in itertools.product(range(waves_n), range(tn), range(mi)):
-        assert col_of_row(w * wn + bj * mi + lane) == w * wn + (bj // vn) * mi * vn + vn * lane + bj % vn
+        assert col_of_row(w * wn + bj * mi + lane) == w * wn + epilogue_column(bj, lane, mi, tn)
 
 
-@pytest.mark.parametrize("wn,mi", [(32, 32), (64, 32), (128, 32), (256, 32), (16, 16), (32, 16), (64, 16), (128, 16)])
+@pytest.mark.parametrize("wn,mi", WAVE_WIDTHS)
 def test_column_interleave_covers_every_column_once_and_matches_the_epilogue(wn, mi):
-    """B[K, N] operand: a lane reads VN consecutive columns at wn0 + v*MI*VN + VN*lane and element e of that
-    read feeds block v*VN + e; the epilogue stores block bj's accumulator to column (bj//VN)*MI*VN + VN*lane + bj%VN."""
-    assert "wn0 + VN * lr;  // + (kk+t)*LDB_S + v*MI*VN" in TEMPLATE and "const int col = wn0 + v * MI * VN + VN * lr;" in TEMPLATE
+    """B[K, N] operand: for a segment (b0, w) a lane reads w consecutive columns at wn0 + b0*MI + w*lane and
+    element e of that read feeds block b0 + e; the epilogue stores that block's accumulator to the same column."""
+    assert "f.b4[t][v] = *(const v4f*)&row[4 * v * MI + 4 * lr];" in TEMPLATE
+    assert "f.b2[t] = *(const v2f*)&row[4 * NSEG4 * MI + 2 * lr];" in TEMPLATE and "f.b1[t] = row[(TN - 1) * MI + lr];" in TEMPLATE
+    assert "const int col = wn0 + b0 * MI + sw * lr;" in TEMPLATE
     tn = wn // mi
-    vn = 4 if tn >= 4 else tn
-    nvb = tn // vn
     fed = {}                                        # (block, lane) -> column whose B values the block's MFMA receives
-    for v, lane, e in itertools.product(range(nvb), range(mi), range(vn)):
-        fed[(v * vn + e, lane)] = v * mi * vn + vn * lane + e
+    for (b0, w), lane in itertools.product(segments(tn), range(mi)):
+        for e in range(w):
+            fed[(b0 + e, lane)] = b0 * mi + w * lane + e
     assert sorted(fed.values()) == list(range(wn))                  # the wave tile's columns, each exactly once
     for (bj, lane), col in fed.items():
-        assert col == (bj // vn) * mi * vn + vn * lane + bj % vn    # where the epilogue writes that accumulator
-    # a lane's VN stores are adjacent, so they leave as one vector store
-    for v, lane in itertools.product(range(nvb), range(mi)):
-        cols = [fed[(v * vn + e, lane)] for e in range(vn)]
-        assert cols == list(range(cols[0], cols[0] + vn)) and cols[0] % vn == 0
+        assert col == epilogue_column(bj, lane, mi, tn)             # where the epilogue writes that accumulator
+    # a lane's w stores are adjacent and aligned to w, so they leave as one vector store
+    for (b0, w), lane in itertools.product(segments(tn), range(mi)):
+        cols = [fed[(b0 + e, lane)] for e in range(w)]
+        assert cols == list(range(cols[0], cols[0] + w)) and cols[0] % w == 0
 
 
 @pytest.mark.parametrize("mi", [32, 16])
 def test_k_permutation_pairs_the_same_k_on_both_operands(mi):
     """MFMA t of a round contracts k = kk + 4*g + t for lane group g: A takes element t of the 128-bit read at
     k offset 4*g, B is read from row kk + 4*g + t; over the 4 MFMAs and 64/mi groups every k of the round once."""
-    assert "const int b_frag = (4 * lg) * LDB_S + wn0 + VN * lr;" in TEMPLATE and "f.b[t][v] = *(const bvec_t*)&Bs[b_frag + (kk + t) * LDB_S" in TEMPLATE
+    assert "const int b_frag = (4 * lg) * LDB_S + wn0;" in TEMPLATE and "const float* row = &Bs[b_frag + (kk + t) * LDB_S];" in TEMPLATE
     kg = 64 // mi
     ksuper = 4 * kg
     seen = []

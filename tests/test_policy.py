@@ -281,19 +281,21 @@ def test_split_block_over_waves():
     assert analyze.split_block_over_waves([64, 64], 4, 8, a) == ([32, 32], 32)   # k step 8 rules out 16x16x4 only
 
 
-def test_mi355x_block_sizes_aim_for_two_waves_per_simd():
+def test_mi355x_block_sizes_aim_for_one_wave_per_simd():
     cfg = MatmulConfig(4096, 8192, 4096, 32)
     policy = Policy(cfg, MI355X())
     td = TileDict.from_block_tile([256, 256], 32, cfg, MI355X())
-    assert policy.recommend_block_size(td)[:3] == [512, 256, 1024]      # 8 waves, then 4 and 16 (tie: smaller first)
+    assert policy.recommend_block_size(td)[:3] == [256, 512, 1024]      # 4 waves, then 8 and 16: whole waves on every SIMD first
+    assert policy.score_block_size(192) > policy.score_block_size(512)  # three waves leave a SIMD idle
     assert Policy(cfg, CUDA()).recommend_block_size(TileDict.from_block_tile([128, 128], 32, cfg, CUDA()))[0] == 128
     hints = get_roller_hints(cfg, MI355X(), topk=4)
     # one block tile at two block sizes, then the next tile.  The 16x16x4 shape is out for both: at
-    # eight waves its 4 x 8 blocks need more fragment registers than half a SIMD's file leaves, at
-    # four waves 128x128 would be 64 blocks, more than the kernel keeps in registers
+    # four waves 128x128 would be 64 blocks, more than the kernel keeps in registers; two waves
+    # of 128x256 hold more accumulators than a lane has registers, so the second size is eight
+    # waves, where 4 x 8 blocks of 16x16 need more fragment registers than half a SIMD's file leaves
     assert [(h.block_tile, h.wave_tile, h.threads, h.mfma) for h in hints] == [
-        ([256, 256], [64, 128], 512, 32), ([256, 256], [128, 128], 256, 32),
-        ([128, 512], [64, 128], 512, 32), ([128, 512], [128, 128], 256, 32)]
+        ([256, 256], [128, 128], 256, 32), ([256, 256], [64, 128], 512, 32),
+        ([128, 512], [128, 128], 256, 32), ([128, 512], [64, 128], 512, 32)]
     assert analyze.split_block_over_waves([256, 256], 4, 32, MI355X(), shapes=[(16, 16, 4)]) is None
     assert analyze.split_block_over_waves([256, 128], 4, 32, MI355X(), shapes=[(16, 16, 4)]) == ([64, 128], 16)   # 4 x 8 = 32 blocks
 
@@ -354,7 +356,10 @@ def test_mi355x_top_hints_compile_without_spills_or_scratch():
 def test_mi355x_small_wave_tiles_list_the_long_k_instruction_first():
     arch = MI355X()
     first = lambda shape: get_roller_hints(MatmulConfig(*shape, 32), arch, topk=2)
-    a, b = first((2048, 2048, 2048))                       # 128x128 over eight waves: 32x64 wave tiles
-    assert (a.wave_tile, a.mfma, b.wave_tile, b.mfma) == ([32, 64], 16, [32, 64], 32)
-    a, b = first((4096, 8192, 4096))                       # 64x128 and larger: 32x32x2 first
-    assert a.mfma == 32 and b.mfma == 32 and a.wave_tile == [64, 128]
+    a, b = first((2048, 2048, 2048))                       # 128x128 over four, then eight waves
+    assert (a.wave_tile, a.mfma, b.wave_tile, b.mfma) == ([64, 64], 16, [32, 64], 16)
+    a, b = first((4096, 8192, 4096))                       # 128x128 wave tiles do not fit 16x16x4 (64 blocks)
+    assert a.mfma == 32 and b.mfma == 32 and a.wave_tile == [128, 128]
+    both = Policy(MatmulConfig(2048, 4096, 2048, 32), arch)._assign_wave_tiles(
+        TileDict.from_block_tile([128, 256], 32, MatmulConfig(2048, 4096, 2048, 32), arch), 256)
+    assert [(t.wave_tile, t.mfma) for t in both] == [([64, 128], 16), ([64, 128], 32)]   # up to 64x128: long k first
