@@ -130,7 +130,7 @@ class MI355X(TileDevice):
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
     # (a test refits it): about 0.95 for 256x256 tiles, 0.81 for 32x64
-    mfma_efficiency: Tuple[float, float] = (0.992, 2.73)
+    mfma_efficiency: Tuple[float, float] = (0.981, 2.07)
     tile_fixed_seconds: float = 1.0e-6
     # 16x16x4 moves half as many accumulator bytes per FLOP as 32x32x2, which leaves the register
     # file free for LDS fragment reads: it wins on every wave tile it fits (up to 64x128; a wave

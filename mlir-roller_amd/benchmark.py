@@ -40,6 +40,11 @@ README_SHAPES: List[Tuple[int, int, int]] = [
 ]
 
 
+# Off the headline table: the ragged named configuration and cubes that put one small tile on a CU
+MID_SHAPES: List[Tuple[int, int, int]] = [(3000, 5000, 1536), (1024, 1024, 1024), (1000, 1000, 1000), (1536, 1536, 1536),
+                                          (1024, 4096, 1024), (16384, 1024, 1024), (6144, 6144, 6144)]
+
+
 def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = DEFAULT_TOPK,
               arch: Optional[TileDevice] = None, baseline: bool = True,
               csv_path: Optional[os.PathLike] = "benchmark_results.csv",
@@ -214,8 +219,9 @@ def plot_results(df: pd.DataFrame, path: os.PathLike, peak_tflops: float = 157.3
 
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(description="Roller fp32 GEMM sweep on MI355X")
-    ap.add_argument("--shapes", default="readme", choices=["readme", "full"],
-                    help="readme: M0..M13; full: all 27 products of {2048,4096,8192}")
+    ap.add_argument("--shapes", default="readme",
+                    help="readme: M0..M13; full: all 27 products of {2048,4096,8192}; mid: the ragged named configuration and "
+                         "mid-size cubes; or a comma-separated list of MxNxK")
     ap.add_argument("--topk", type=int, default=DEFAULT_TOPK, help="hints tried per shape (the reference tries 20)")
     ap.add_argument("--no-baseline", action="store_true")
     ap.add_argument("--csv", default="benchmark_results.csv")
@@ -228,8 +234,17 @@ def main(argv=None) -> None:
     if args.shapes == "full":
         dims = [2048, 4096, 8192]
         shapes = list(itertools.product(dims, dims, dims))
-    else:
+    elif args.shapes == "mid":
+        shapes = list(MID_SHAPES)
+    elif args.shapes == "readme":
         shapes = README_SHAPES
+    else:
+        try:
+            shapes = [tuple(int(v) for v in item.lower().split("x")) for item in args.shapes.split(",")]
+            if any(len(sh) != 3 or min(sh) <= 0 for sh in shapes):
+                raise ValueError
+        except ValueError:
+            ap.error(f"--shapes {args.shapes}: expected readme, full, mid or a comma-separated list of MxNxK")
     df = benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump,
                    counters=args.counters, vendor=args.vendor)
     if args.plot:

@@ -363,3 +363,49 @@ def test_mi355x_small_wave_tiles_list_the_long_k_instruction_first():
     both = Policy(MatmulConfig(2048, 4096, 2048, 32), arch)._assign_wave_tiles(
         TileDict.from_block_tile([128, 256], 32, MatmulConfig(2048, 4096, 2048, 32), arch), 256)
     assert [(t.wave_tile, t.mfma) for t in both] == [([64, 128], 16), ([64, 128], 32)]   # up to 64x128: long k first
+
+
+def test_committed_ranking_constants_equal_a_refit_of_the_committed_sweep():
+    """The MI355X ranking model is reproducible from the tree: refitting the committed sweep gives
+    the constants that ``arch.MI355X`` carries, and replaying the policy on that sweep finds a kernel
+    within half a percent of the fastest measured one among its first four hints on every
+    benchmark shape."""
+    from mlir_roller_amd import calibrate
+    data = calibrate.load()
+    records = data["records"]
+    assert len(records) >= 500 and len({tuple(r["shape"]) for r in records}) >= 15
+    arch = MI355X()
+    fit = calibrate.fit(records)
+    assert tuple(fit["mfma_efficiency"]) == tuple(arch.mfma_efficiency), fit
+    assert fit["rms_residual"] < 0.02 and fit["points"] >= 100
+    assert calibrate.fit_waves_per_simd(records)["waves_per_partition"] == arch.waves_per_partition
+    assert calibrate.fit_long_k_mfma(records)["long_k_mfma_up_to"] == arch.long_k_mfma_up_to
+    from mlir_roller_amd.benchmark import README_SHAPES
+    rows = {tuple(r["shape"]): r for r in calibrate.check(records, topk=4)}
+    for shape in list(README_SHAPES) + [(3000, 5000, 1536)]:
+        row = rows[shape]
+        assert row["unmeasured_in_topk"] == 0 and row["topk_over_fastest"] <= 1.005, row
+        assert row["top1_over_fastest"] <= 1.01, row
+
+
+def test_refit_rejects_a_sweep_that_cannot_pin_the_model():
+    from mlir_roller_amd import calibrate
+    with pytest.raises(ValueError):
+        calibrate.fit([])
+    one = [{"shape": [4096, 4096, 4096], "block_tile": [256, 256], "wave_tile": [128, 128], "mfma": 32, "rstep": 32,
+            "threads": 256, "ms": 0.95}]
+    with pytest.raises(ValueError):
+        calibrate.fit(one)
+    with pytest.raises(ValueError):
+        calibrate.fit_waves_per_simd(one)
+    # a synthetic sweep that follows the model exactly is recovered exactly
+    arch = MI355X()
+    synth = []
+    for m, n in [(256, 256), (128, 256), (128, 128), (64, 128), (64, 64), (32, 64)]:
+        eff = 0.95 - 2.5 * (1 / m + 1 / n)
+        per_cu = (4096 // m) * (4096 // n) // 256
+        t = per_cu * (calibrate.ideal_tile_seconds(m, n, 4096, 32, arch) / eff + calibrate.fixed_tile_seconds(m, n, arch))
+        synth.append({"shape": [4096, 4096, 4096], "block_tile": [m, n], "wave_tile": [m // 2, n // 2], "mfma": 16,
+                      "rstep": 32, "threads": 256, "ms": t * 1e3})
+    got = calibrate.fit(synth)
+    assert got["mfma_efficiency"] == (0.95, 2.5) and got["rms_residual"] < 1e-9
