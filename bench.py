@@ -140,21 +140,35 @@ def copy_workload(args) -> int:
     return 0 if ok else 1
 
 
+def traffic_key(kernel_tag: str) -> str:
+    """The part of a kernel's tag that decides its HBM-side traffic: block tile, K step, depth,
+    layout and workgroup order -- not how the block tile is split over waves or which matrix
+    instruction multiplies it."""
+    import re
+    return re.sub(r"_w\d+x\d+_mi\d+", "", kernel_tag)
+
+
 def measured_traffic(workload: str, kernels: dict):
-    """(bytes per launch, note) from the committed counter summary, or (None, reason)."""
+    """(bytes per launch, note) from the committed counter summary, or (None, reason).  The summary
+    holds, per workload and shape, the bytes one launch moved and the kernel it was measured with;
+    the figure is used only if every shape of this run kept a kernel with the same traffic key."""
     try:
         table = json.loads(TRAFFIC_FILE.read_text())
     except Exception:
         return None, f"{TRAFFIC_FILE.name} not found"
     entry = table.get(workload)
+    if not entry and set(kernels) <= set(table.get("sweep", {}).get("per_shape", {})):
+        entry = table["sweep"]   # a single shape of the sweep: its row of the sweep's counter run
     if not entry:
         return None, f"no counter run recorded for workload {workload!r}"
-    recorded = entry.get("kernels", {})
-    differing = sorted(k for k in kernels if recorded.get(k) != kernels[k])
+    per_shape = entry.get("per_shape", {})
+    differing = sorted(k for k, tag in kernels.items()
+                       if k not in per_shape or traffic_key(per_shape[k]["kernel"]) != traffic_key(tag))
     if differing:
-        return None, ("counter run was taken with other kernels for " + ", ".join(differing[:4])
+        return None, ("counter run was taken with other block tiles for " + ", ".join(differing[:4])
                       + ("..." if len(differing) > 4 else ""))
-    return float(entry["traffic_bytes_per_launch"]), entry.get("source", "")
+    total = sum(per_shape[k]["traffic_bytes"] for k in kernels)
+    return float(total) / len(kernels), entry.get("source", "")
 
 
 def main() -> int:
