@@ -28,8 +28,10 @@
 //               LDS buffers, so that loads run two and three K steps ahead of the MFMAs -- for
 //               short K steps whose MFMA time does not cover a trip to HBM
 //   PAD_A,PAD_B extra floats per LDS row of the A tile ([BM][BK+PAD_A]) and B tile ([BK][BN+PAD_B])
-//   VEC         4 = 128-bit global accesses (needs K%4==0, N%4==0, lda/ldb/ldc%4==0 and 16-byte
-//               aligned base pointers), 1 = dword accesses with per-element predicates
+//   VEC         4 = 16-byte aligned 128-bit global accesses (needs K%4==0, N%4==0, lda/ldb/ldc%4==0
+//               and 16-byte aligned base pointers), 1 = any K, N, leading dimension and 4-byte
+//               aligned pointers: 128-bit loads at dword alignment with per-element zeroing of
+//               what lies past a row's end, dword stores
 //   EDGE        1 = predicate ragged tiles (any M, N, K), 2 = M and N may be ragged but the host
 //               guarantees BK|K (no per-step K predicates), 0 = host guarantees BM|M, BN|N, BK|K
 //   SWZ         workgroup-id remap: bit0 = give every XCD a contiguous run of tiles,
@@ -264,11 +266,14 @@ DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool
   (void)p1; (void)p2; (void)p3;
   return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, p0 ? off : OOB_OFFSET, 0, 0));
 #else
-  v4f v;
-  v.x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p0 ? off : OOB_OFFSET, 0, 0));
-  v.y = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p1 ? off + 4 : OOB_OFFSET, 0, 0));
-  v.z = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p2 ? off + 8 : OOB_OFFSET, 0, 0));
-  v.w = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, p3 ? off + 12 : OOB_OFFSET, 0, 0));
+  // Rows that are not multiples of four floats long start at dword-aligned addresses only.  The
+  // four elements still come with one 128-bit load (the memory pipeline accepts dword alignment
+  // for multi-dword buffer loads); elements past the end of a row or column range would carry the
+  // neighbouring row's data and are zeroed here.  The predicates are monotone (p0 >= p1 >= p2 >= p3).
+  v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, p0 ? off : OOB_OFFSET, 0, 0));
+  v.y = p1 ? v.y : 0.0f;
+  v.z = p2 ? v.z : 0.0f;
+  v.w = p3 ? v.w : 0.0f;
   return v;
 #endif
 }
