@@ -107,6 +107,26 @@ extern "C" __global__ __launch_bounds__(256) void clock_probe(long long* out, fl
 """
 
 
+# Engine clock under the GEMM load itself: one wave on a second stream sleeps and samples the two
+# counters while the timed steps run; it ends after `ticks` of the 100 MHz counter or `max_iters`
+# samples, whichever comes first.
+SAMPLER_KERNEL = r"""
+extern "C" __global__ void clock_sampler(long long* out, long long ticks, int max_iters) {
+  const long long r0 = __builtin_amdgcn_s_memrealtime();
+  const long long c0 = __builtin_readcyclecounter();
+  long long r = r0, c = c0;
+  int it = 0;
+  while (r - r0 < ticks && it < max_iters) {
+    __builtin_amdgcn_s_sleep(64);
+    r = __builtin_amdgcn_s_memrealtime();
+    c = __builtin_readcyclecounter();
+    ++it;
+  }
+  if (threadIdx.x == 0) { out[0] = c - c0; out[1] = r - r0; out[2] = it; }
+}
+"""
+
+
 def copy_workload(args) -> int:
     """Calibration workload for the HBM traffic counters: a plain copy of 256 MiB per launch
     (256 MiB read, 256 MiB written), so that FETCH_SIZE / WRITE_SIZE of the GEMM kernel can be
@@ -347,7 +367,7 @@ def main() -> int:
         ms = dict(timings).get(rank, float("nan"))
         log(f"[bench] {name} {shape}: rank {rank}/{len(hints)} {g.tag()}  {ms:.4f} ms  "
             f"{2.0 * M * N * K / ms / 1e9:.1f} TFLOP/s  normwise {rep['normwise']:.2e} max_abs {rep['max_abs']:.2e}  {summary}")
-        return {"name": name, "shape": shape, "plan": plan, "bufs": bufs, "rank": rank, "hints": len(hints),
+        return {"name": name, "shape": shape, "plan": plan, "bufs": bufs, "rank": rank, "hints": len(hints), "tuned_ms": ms,
                 "summary": summary, "cfg": g, "hint": text, "rep": rep, "host_ms": t_host * 1e3, "dist": distribution}
 
     cases = []
@@ -374,6 +394,14 @@ def main() -> int:
         clock_probe = probe_mod.get_function("clock_probe")
         probe_waves = 4 * props.compute_units   # one workgroup of four waves per CU: one wave per SIMD
         probe_out, probe_sink = DeviceArray((2 * probe_waves,), np.int64), DeviceArray((probe_waves,))
+        sampler_mod = Module(hip.compile_source(SAMPLER_KERNEL, "clock_sampler.hip")[0])
+        clock_sampler = sampler_mod.get_function("clock_sampler")
+        sampler_out = DeviceArray.zeros((4,), np.int64)
+        side_stream = Stream()
+        # sample for about 70 % of what the timed steps should take (tuned times; 1 ms at least)
+        expect_ms = args.steps * sum(c["tuned_ms"] if c["tuned_ms"] == c["tuned_ms"] else 2.0 * c["shape"][0] * c["shape"][1] * c["shape"][2] / 120e9
+                                     for c in cases)
+        sampler_ticks = int(max(1.0, 0.7 * expect_ms) * 1e5)       # 100 MHz: 1e5 ticks per millisecond
     hip.synchronize()
     step_est_ms = sum(2.0 * s[0] * s[1] * s[2] for s in shapes) / 120e9
     for _ in range(max(args.warmup, int(tuner.RAMP_MS / step_est_ms) + 1)):
@@ -381,6 +409,8 @@ def main() -> int:
     e0, e1 = Event(), Event()
     wall0 = time.perf_counter()
     e0.record(stream)
+    if clock_probe is not None:
+        clock_sampler((1,), (64,), (sampler_out, ctypes.c_longlong(sampler_ticks), max(1000, sampler_ticks // 20)), stream=side_stream)
     for _ in range(args.steps):
         one_step()
     e1.record(stream)
@@ -392,10 +422,15 @@ def main() -> int:
     wall_ms = (time.perf_counter() - wall0) * 1e3
     total_ms = hip.get_elapsed_time(e0, e1)
     ms_per_step = total_ms / max(args.steps, 1)
-    achieved_mhz = None
+    achieved_mhz = probe_mhz = None
+    sampler_ms = None
     if clock_probe is not None:
         ticks = probe_out.get().reshape(-1, 2).astype(np.float64)
-        achieved_mhz = round(float(np.median(ticks[:, 0] / np.maximum(ticks[:, 1], 1.0))) * 100.0, 1)
+        probe_mhz = round(float(np.median(ticks[:, 0] / np.maximum(ticks[:, 1], 1.0))) * 100.0, 1)
+        cycles, real, _samples, _ = (int(v) for v in sampler_out.get())
+        if real > 0:
+            achieved_mhz = round(cycles / real * 100.0, 1)
+            sampler_ms = round(real / 1e5, 3)
 
     # per-shape timing of the winners (outside the headline region)
     per_shape = []
@@ -495,8 +530,10 @@ def main() -> int:
         "tune_s": round(timers["tune_s"], 3), "tuned_from_cache": from_cache_shapes == prepared_shapes,
         "verify_s": round(timers["verify_s"], 3),
         "device": {"name": device_name, "arch": props.arch.decode(), "compute_units": props.compute_units,
-                   "clock_mhz": props.clock_khz // 1000, "achieved_clock_mhz": achieved_mhz,
-                   "achieved_clock_note": "shader cycle counter over the 100 MHz constant counter in an MFMA probe kernel queued directly behind the timed steps"},
+                   "clock_mhz": props.clock_khz // 1000, "achieved_clock_mhz": achieved_mhz, "achieved_clock_window_ms": sampler_ms,
+                   "mfma_probe_clock_mhz": probe_mhz,
+                   "achieved_clock_note": "shader cycle counter over the 100 MHz constant counter: achieved = one sampling wave on a second "
+                                          "stream while the timed steps run; mfma_probe = a pure-MFMA kernel queued directly behind them"},
         "named_configs": named,
         "per_shape": per_shape,
     }

@@ -202,3 +202,13 @@ def test_concurrent_precompiles_and_thread_local_errors(hip_lib, tmp_path):
             assert f.read_bytes()[:4] == b"\x7fELF" and f.read_bytes()[-16:-12] == b"RLHC"
     finally:
         hip.set_cache_dir(hip.DEFAULT_CACHE_DIR)
+
+
+def test_lds_requests_beyond_a_cu_are_refused_without_a_device(hip_lib):
+    # more dynamic LDS than a CU has: refused with text before anything reaches the runtime
+    assert hip_lib.rl_func_set_max_dynamic_lds(C.c_void_p(1), 160 * 1024 + 4) == hip.RL_ERR_INVALID_ARG
+    assert b"exceed the 160 KB" in hip_lib.rl_last_error()
+    assert hip_lib.rl_func_set_max_dynamic_lds(None, 1024) == hip.RL_ERR_INVALID_ARG
+    with pytest.raises(HipError, match="exceed the 160 KB"):
+        hip.config_check(GemmConfig(256, 256, 48, 128, 128, 32, 2, 0, 0, 4, 1))       # 2 x 96 KB
+    assert hip_lib.rl_gemm_plan_lds_limit(None) == 0 and hip_lib.rl_gemm_plan_lds_bytes(None) == 0

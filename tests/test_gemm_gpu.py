@@ -414,6 +414,35 @@ def test_lds_grant_is_read_back_and_large_tiles_launch(device):
         fn((1,), (256,), (DeviceArray((4,)),) * 3 + (0, 0, 0, 0, 0, 0), shared_mem=device.lds_bytes_per_block + 1024)
 
 
+def test_calls_from_another_thread_use_the_initialised_device(device):
+    # the current device is per-thread state of the runtime: every entry point selects it again
+    import threading
+    cfg = GemmConfig(128, 128, 32, 64, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1)
+    A, B = go.make_inputs(200, 300, 96, seed=11, distribution="integer")
+    out = {}
+
+    def worker():
+        try:
+            out["C"] = run_gemm(cfg, A, B)          # malloc, memcpy, plan launch, sync, free on this thread
+            e0, e1 = hip.Event(), hip.Event()
+            e0.record(); e1.record(); e1.synchronize()
+            out["ms"] = hip.get_elapsed_time(e0, e1)
+        except Exception as e:                       # surfaced in the main thread below
+            out["error"] = e
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join(60)
+    assert not t.is_alive() and "error" not in out, out.get("error")
+    assert np.array_equal(out["C"], go.gemm_f32(A, B)) and out["ms"] >= 0.0
+    # clearing the plans waits for the device and for launch calls in progress; old handles are refused afterwards
+    plan = GemmPlan(cfg)
+    hip.check(hip.lib().rl_gemm_plans_clear())
+    with pytest.raises(HipError, match="released"):
+        plan.launch(DeviceArray((4,)), DeviceArray((4,)), DeviceArray((4,)), 1, 4, 4)
+    assert np.array_equal(run_gemm(cfg, A, B), go.gemm_f32(A, B))     # a fresh plan works
+
+
 def test_low_level_module_api_like_the_reference_uses_cupy(device):
     src = r'''extern "C" __global__ void axpy(float a, const float* x, float* y, int n) {
         int i = blockIdx.x * blockDim.x + threadIdx.x;
