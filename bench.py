@@ -483,11 +483,25 @@ def main() -> int:
     # ---- cold JIT cost: hiprtc on every kernel a first run compiles, every cache bypassed ----------
     compile_cold = None
     if not args.lean:
+        # the compiler library keeps a cache of its own on disk (AMD_COMGR_CACHE_DIR, on by default):
+        # point it at an empty directory for this phase, or "cold" would be a lookup
+        import shutil
+        import tempfile
+        scratch_dir = tempfile.mkdtemp(prefix="roller_cold_jit_")
+        previous = os.environ.get("AMD_COMGR_CACHE_DIR")
+        os.environ["AMD_COMGR_CACHE_DIR"] = scratch_dir
         t_unique = {}
-        for g in candidates_seen:
-            t0 = time.perf_counter()
-            hip.compile_config(g)
-            t_unique[g] = time.perf_counter() - t0
+        try:
+            for g in candidates_seen:
+                t0 = time.perf_counter()
+                hip.compile_config(g)
+                t_unique[g] = time.perf_counter() - t0
+        finally:
+            if previous is None:
+                os.environ.pop("AMD_COMGR_CACHE_DIR", None)
+            else:
+                os.environ["AMD_COMGR_CACHE_DIR"] = previous
+            shutil.rmtree(scratch_dir, ignore_errors=True)
         compile_cold = {"unique_kernels": len(t_unique), "unique_s": round(sum(t_unique.values()), 2),
                         "per_shape_hint_pairs": len(pairs_seen), "pairs_s": round(sum(t_unique[g] for g in pairs_seen), 2)}
 
