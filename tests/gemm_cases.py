@@ -28,3 +28,56 @@ def seeded_policy_cases(arch, count: int = 40, seed: int = 20240607):
         if not hints:
             raise AssertionError(f"no hints for {(M, N, K)}")
         yield case, config, hints[int(rng.integers(0, len(hints)))], depth, trans_b, accumulate
+
+
+def seeded_template_cases(count: int = 72, seed: int = 20250101):
+    """Yields ``(case, GemmConfig, (M, N, K))``: random points of the kernel template's own
+    parameter space -- not what the policy would pick -- with a problem size to match: both matrix
+    instructions, 1 to 8 waves, 1 to 7 column blocks per wave, K steps of 1 to 8 fragment rounds,
+    every pipeline depth, layout, edge mode, access width, remap mode and padding the library
+    accepts.  Only configurations that ``rl_gemm_config_check`` accepts are kept."""
+    from mlir_roller_amd import hip
+    from mlir_roller_amd.hip import GemmConfig
+
+    rng = np.random.default_rng(seed)
+    pick = lambda options: options[int(rng.integers(0, len(options)))]
+    case = 0
+    while case < count:
+        mi = pick([16, 32])
+        tm, tn = int(rng.integers(1, 5)), int(rng.integers(1, 8))
+        waves_m, waves_n = pick([1, 1, 2, 4]), pick([1, 2, 2, 4])
+        acc_regs = tm * tn * (16 if mi == 32 else 4)
+        if tm * tn > 32 or waves_m * waves_n > 8 or acc_regs > (128 if waves_m * waves_n > 4 else 256):
+            continue
+        wm, wn = tm * mi, tn * mi
+        bm, bn = wm * waves_m, wn * waves_n
+        if bm > 384 or bn > 448:
+            continue
+        bk = (4 * 64 // mi) * pick([1, 1, 2, 2, 3, 4, 8])
+        vec, trans_b, accum = pick([4, 4, 1]), pick([0, 0, 1]), pick([0, 0, 1])
+        stages = pick([1, 2, 3, 3, 4, 4, 5, 5])
+        threads = 64 * waves_m * waves_n
+        a_units, b_units = bm * bk // 4, bk * bn // 4
+        can_direct = stages >= 3 and vec == 4 and bk & (bk - 1) == 0 and a_units % 64 == 0 and b_units % 64 == 0
+        direct = int(can_direct and rng.random() < 0.8)
+        if stages > 3 and not (direct and a_units % threads == 0 and b_units % threads == 0):
+            stages = 3
+        pad_a = 0 if direct else pick([0, 4])
+        pad_b = 0 if direct else pick([0, 0, 4])
+        swz, group = pick([0, 1, 2, 3, 3]), pick([1, 3, 8])
+        M, N, K = int(rng.integers(1, 3 * bm)), int(rng.integers(1, 3 * bn)), int(rng.integers(1, 5 * bk + 1))
+        if rng.random() < 0.3:
+            M, N, K = -(-M // bm) * bm, -(-N // bn) * bn, -(-K // bk) * bk           # sometimes whole tiles
+        elif rng.random() < 0.4:
+            K = -(-K // bk) * bk                                                      # only M and N ragged
+        if vec == 4:
+            N, K = max(4, N // 4 * 4), max(4, K // 4 * 4)
+        aligned_mn, aligned_k = M % bm == 0 and N % bn == 0, K % bk == 0
+        edge = 1 if not aligned_k else (2 if not aligned_mn else pick([0, 0, 1, 2]))
+        cfg = GemmConfig(bm, bn, bk, wm, wn, mi, stages, pad_a, pad_b, vec, edge, swz, group, accum, direct, trans_b)
+        try:
+            hip.config_check(cfg)
+        except hip.HipError:
+            continue
+        yield case, cfg, (M, N, K)
+        case += 1
