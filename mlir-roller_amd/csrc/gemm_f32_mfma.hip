@@ -261,6 +261,7 @@ DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* base, long bytes) {
   return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, n, 0x00020000);
 }
 
+template <bool SAME = false>
 DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool p2, bool p3) {
 #if VEC == 4
   (void)p1; (void)p2; (void)p3;
@@ -269,11 +270,14 @@ DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool
   // Rows that are not multiples of four floats long start at dword-aligned addresses only.  The
   // four elements still come with one 128-bit load (the memory pipeline accepts dword alignment
   // for multi-dword buffer loads); elements past the end of a row or column range would carry the
-  // neighbouring row's data and are zeroed here.  The predicates are monotone (p0 >= p1 >= p2 >= p3).
+  // neighbouring row's data and are zeroed here.  The predicates are monotone (p0 >= p1 >= p2 >= p3);
+  // SAME says that the caller passes four equal ones (the unit is in or out as a whole).
   v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, p0 ? off : OOB_OFFSET, 0, 0));
-  v.y = p1 ? v.y : 0.0f;
-  v.z = p2 ? v.z : 0.0f;
-  v.w = p3 ? v.w : 0.0f;
+  if constexpr (!SAME) {
+    v.y = p1 ? v.y : 0.0f;
+    v.z = p2 ? v.z : 0.0f;
+    v.w = p3 ? v.w : 0.0f;
+  }
   return v;
 #endif
 }
@@ -419,7 +423,10 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #if DIRECT
   // Issues the loads of K step kt straight into LDS buffer `stage`.  Instruction i of a wave
   // fills the 64 consecutive 16-byte units that start at unit i*NT + wave*64 of the operand tile.
-  auto fetch_direct = [&](int kt, int stage) {
+  // KTAIL (a compile-time 0/1) says whether tile kt may be the one that K ends in: only then are
+  // the units tested against K.
+  auto fetch_direct = [&](auto ktail, int kt, int stage) {
+    constexpr bool KTEST = EDGE_K && decltype(ktail)::value;
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
     const int k0 = kt * BK;
     const bool live = kt < KT;
@@ -431,7 +438,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < A_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (A_UNITS % NT == 0 || first < A_UNITS) {
-        const bool ok = a_ok[i] && (!EDGE_K || k0 + a_kcol[i] < K);
+        const bool ok = a_ok[i] && (!KTEST || k0 + a_kcol[i] < K);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr_t)(As + first * 4), 16, ok ? a_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -439,7 +446,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < B_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (B_UNITS % NT == 0 || first < B_UNITS) {
-        const bool ok = b_ok[i][0] && (!EDGE_K || k0 + b_krow[i] < K);  // K % 4 == 0: a chunk is in or out as a whole
+        const bool ok = b_ok[i][0] && (!KTEST || k0 + b_krow[i] < K);  // K % 4 == 0: a chunk is in or out as a whole
         __builtin_amdgcn_raw_ptr_buffer_load_lds(br, (lds_ptr_t)(Bs + first * 4), 16, ok ? b_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -448,8 +455,10 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 
   // Issues the global loads of K step kt into the staging registers.  A step at or beyond KT
   // (the pipelined loop asks for up to two steps ahead) gets an empty resource: every load
-  // returns 0 and touches no memory.
-  auto fetch = [&](int kt) {
+  // returns 0 and touches no memory.  KTAIL (a compile-time 0/1) says whether tile kt may be the
+  // one that K ends in: only then are the elements tested against K.
+  auto fetch = [&](auto ktail, int kt) {
+    constexpr bool KTEST = EDGE_K && decltype(ktail)::value;
     const int k0 = kt * BK;
     const bool live = kt < KT;
     const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, live ? a_rem - (long)k0 * 4 : 0);
@@ -457,21 +466,21 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
     for (int i = 0; i < A_PER_T; ++i) {
       const int k = k0 + a_kcol[i];
-      ra[i] = load_unit(ar, a_goff[i],
-                        a_ok[i] && (!EDGE_K || k + 0 < K), a_ok[i] && (!EDGE_K || k + 1 < K),
-                        a_ok[i] && (!EDGE_K || k + 2 < K), a_ok[i] && (!EDGE_K || k + 3 < K));
+      ra[i] = load_unit<!KTEST>(ar, a_goff[i],
+                                a_ok[i] && (!KTEST || k + 0 < K), a_ok[i] && (!KTEST || k + 1 < K),
+                                a_ok[i] && (!KTEST || k + 2 < K), a_ok[i] && (!KTEST || k + 3 < K));
     }
 #pragma unroll
     for (int i = 0; i < B_PER_T; ++i) {
 #if TRANS_B
       const int k = k0 + b_krow[i];
-      rb[i] = load_unit(br, b_goff[i],
-                        b_ok[i][0] && (!EDGE_K || k + 0 < K), b_ok[i][1] && (!EDGE_K || k + 1 < K),
-                        b_ok[i][2] && (!EDGE_K || k + 2 < K), b_ok[i][3] && (!EDGE_K || k + 3 < K));
+      rb[i] = load_unit<!KTEST>(br, b_goff[i],
+                                b_ok[i][0] && (!KTEST || k + 0 < K), b_ok[i][1] && (!KTEST || k + 1 < K),
+                                b_ok[i][2] && (!KTEST || k + 2 < K), b_ok[i][3] && (!KTEST || k + 3 < K));
 #else
-      const bool kin = !EDGE_K || k0 + b_krow[i] < K;
-      rb[i] = load_unit(br, b_goff[i], b_ok[i][0] && kin, b_ok[i][1] && kin, b_ok[i][2] && kin,
-                        b_ok[i][3] && kin);
+      const bool kin = !KTEST || k0 + b_krow[i] < K;
+      rb[i] = load_unit<!EDGE>(br, b_goff[i], b_ok[i][0] && kin, b_ok[i][1] && kin, b_ok[i][2] && kin,
+                               b_ok[i][3] && kin);
 #endif
     }
   };
@@ -579,13 +588,13 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     frag_t fr[2];
 #if DIRECT
 #pragma unroll
-    for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(i, i);
+    for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(int_c<1>{}, i, i);
     // this wave's part of tile 0 is in LDS (of every requested tile when the loads per wave differ)
     WAIT_VMCNT(PROLOGUE_IN_FLIGHT);
 #else
-    fetch(0);
+    fetch(int_c<1>{}, 0);
     stash(0);
-    fetch(1);
+    fetch(int_c<1>{}, 1);
 #endif
     __syncthreads();
     read_frags(fr[0], 0, 0);
@@ -595,7 +604,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // MFMAs and fragment reads per round; LDS writes and global loads per K step
     constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NSEG), W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
 
-    auto step = [&](auto parity, int kt) {
+    auto step = [&](auto parity, auto ktail, int kt) {
       constexpr int P = decltype(parity)::value;
       const int cur = (unsigned)kt % LDS_BUFS, nxt = (unsigned)(kt + 1) % LDS_BUFS;
 #pragma unroll
@@ -619,7 +628,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       WAIT_VMCNT((LDS_BUFS - 2) * LOADS_PER_TILE);
       __syncthreads();
       read_frags(fr[(P + SUPERS) & 1], nxt, 0);
-      fetch_direct(kt + LDS_BUFS, cur);
+      fetch_direct(ktail, kt + LDS_BUFS, cur);
       mfma_frags(fr[(P + SUPERS - 1) & 1], 1, 4);
 #if SCHED
       {
@@ -635,7 +644,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #else
       mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
       stash(nxt);
-      fetch(kt + 2);
+      fetch(ktail, kt + 2);
 #if SCHED
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
@@ -668,22 +677,35 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
     };
 
-    int kt = 0;
-    if constexpr (SUPERS % 2 == 0) {
-      for (; kt < KT - 1; ++kt) step(int_c<0>{}, kt);
-      last_step(int_c<0>{}, kt);
-    } else {
-      // an odd number of rounds per step flips the parity every step: unroll by two
-      for (; kt + 1 < KT - 1; kt += 2) {
-        step(int_c<0>{}, kt);
-        step(int_c<1>{}, kt + 1);
-      }
-      if (kt < KT - 1) {
-        step(int_c<0>{}, kt);
-        last_step(int_c<1>{}, kt + 1);
+    // Pipelined steps [from, to).  An odd number of rounds per step flips the fragment-set parity
+    // every step, so the parity of a step is that of its index.
+    auto steps = [&](auto ktail, int from, int to) {
+      int kt = from;
+      if constexpr (SUPERS % 2 == 0) {
+        for (; kt < to; ++kt) step(int_c<0>{}, ktail, kt);
       } else {
-        last_step(int_c<0>{}, kt);
+        if (kt < to && (kt & 1)) step(int_c<1>{}, ktail, kt++);
+        for (; kt + 1 < to; kt += 2) {
+          step(int_c<0>{}, ktail, kt);
+          step(int_c<1>{}, ktail, kt + 1);
+        }
+        if (kt < to) step(int_c<0>{}, ktail, kt);
       }
+    };
+    // Step kt requests tile kt + LDS_BUFS.  Only tile KT-1 can be cut short by K, so only the step
+    // that requests it tests its units against K; the steps behind it request tiles past the end
+    // (empty range: zeros whatever the test says) and share its code.
+#if EDGE_K
+    const int plain = KT - 1 - LDS_BUFS > 0 ? KT - 1 - LDS_BUFS : 0;
+    steps(int_c<0>{}, 0, plain);
+    steps(int_c<1>{}, plain, KT - 1);
+#else
+    steps(int_c<0>{}, 0, KT - 1);
+#endif
+    if (SUPERS % 2 == 0 || (KT - 1) % 2 == 0) {
+      last_step(int_c<0>{}, KT - 1);
+    } else {
+      last_step(int_c<1>{}, KT - 1);
     }
   }
 #else
@@ -697,7 +719,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     }
   };
   if (KT > 0) {
-    fetch(0);
+    fetch(int_c<1>{}, 0);
     stash(0);
   }
   __syncthreads();
@@ -705,12 +727,12 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const bool more = kt + 1 < KT;
 #if STAGES == 2
     const int cur = kt & 1;
-    if (more) fetch(kt + 1);
+    if (more) fetch(int_c<1>{}, kt + 1);
     multiply(cur);
     if (more) stash(cur ^ 1);
     __syncthreads();
 #else
-    if (more) fetch(kt + 1);
+    if (more) fetch(int_c<1>{}, kt + 1);
     multiply(0);
     __syncthreads();
     if (more) stash(0);

@@ -362,6 +362,40 @@ def test_results_are_bitwise_reproducible_and_independent_of_tile_order(device):
     assert np.array_equal(first, run_gemm(GemmConfig(128, 128, 32, 64, 64, 32, 2, 4, 0, 4, 1), A, B))
 
 
+K_TAIL_CONFIGS = [
+    GemmConfig(128, 128, 32, 64, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1),        # direct-to-LDS, four rounds per step
+    GemmConfig(128, 128, 8, 64, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1),         # direct-to-LDS, one round per step (parity flips)
+    GemmConfig(128, 128, 32, 64, 64, 16, 5, 0, 0, 4, 1, 3, 8, 0, 1),        # four LDS buffers: the tail is requested three steps ahead
+    GemmConfig(128, 128, 32, 32, 64, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1, 1),     # transposed second operand, direct-to-LDS
+    GemmConfig(128, 128, 16, 64, 64, 32, 3, 4, 0, 4, 1),                    # register-staged, 128-bit accesses
+    GemmConfig(128, 128, 24, 64, 64, 32, 3, 4, 0, 4, 1),                    # register-staged, three rounds per step
+    GemmConfig(128, 128, 16, 64, 64, 16, 3, 4, 4, 1, 1),                    # dword-aligned rows: K and N odd
+    GemmConfig(128, 128, 16, 64, 64, 16, 3, 4, 4, 1, 1, 3, 8, 0, 0, 1),     # the same with the transposed operand
+]
+
+
+@pytest.mark.parametrize("cfg", K_TAIL_CONFIGS, ids=[c.tag() for c in K_TAIL_CONFIGS])
+def test_k_tail_at_every_position_of_the_pipeline(device, cfg):
+    """K ends inside the last K step; only the pipeline step that requests that tile tests its
+    loads against K.  One to seven K steps put that step before the loop, at its start, in its
+    middle and nowhere (fewer steps than buffers).  Exact on integers; and a row of A must not
+    pick up the start of the next row: with NaN in the first column of every odd row, the even
+    rows of C stay finite (a tail read as data and multiplied by the zero rows past the end of
+    B would turn them into NaN)."""
+    M = 130
+    N = 260 if cfg.vec == 4 else 259
+    tails = (4, cfg.bk - 4) if cfg.vec == 4 else (1, cfg.bk - 1)
+    for steps in range(1, 8):
+        for tail in tails:
+            K = (steps - 1) * cfg.bk + tail
+            say("case", cfg.tag(), (M, N, K))
+            Ai, Bi = go.make_inputs(M, N, K, seed=steps + 10 * tail, distribution="integer")
+            assert np.array_equal(run_gemm(cfg, Ai, Bi), go.c_gemm_f32(Ai, Bi)), (steps, tail)
+            Ai[1::2, 0] = np.nan
+            got = run_gemm(cfg, Ai, Bi)
+            assert np.isnan(got[1::2]).all() and np.isfinite(got[0::2]).all(), (steps, tail)
+
+
 def test_pipeline_depth_does_not_change_the_bits(device):
     """Depths 1, 2, 3 and the direct-to-LDS variant run the same MFMAs in the same order per
     accumulator; only the way operands reach LDS differs."""
