@@ -677,6 +677,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
     };
 
+#if EDGE_K
     // Pipelined steps [from, to).  An odd number of rounds per step flips the fragment-set parity
     // every step, so the parity of a step is that of its index.
     auto steps = [&](auto ktail, int from, int to) {
@@ -695,18 +696,33 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // Step kt requests tile kt + LDS_BUFS.  Only tile KT-1 can be cut short by K, so only the step
     // that requests it tests its units against K; the steps behind it request tiles past the end
     // (empty range: zeros whatever the test says) and share its code.
-#if EDGE_K
     const int plain = KT - 1 - LDS_BUFS > 0 ? KT - 1 - LDS_BUFS : 0;
     steps(int_c<0>{}, 0, plain);
     steps(int_c<1>{}, plain, KT - 1);
-#else
-    steps(int_c<0>{}, 0, KT - 1);
-#endif
     if (SUPERS % 2 == 0 || (KT - 1) % 2 == 0) {
       last_step(int_c<0>{}, KT - 1);
     } else {
       last_step(int_c<1>{}, KT - 1);
     }
+#else
+    int kt = 0;
+    if constexpr (SUPERS % 2 == 0) {
+      for (; kt < KT - 1; ++kt) step(int_c<0>{}, int_c<0>{}, kt);
+      last_step(int_c<0>{}, kt);
+    } else {
+      // an odd number of rounds per step flips the parity every step: unroll by two
+      for (; kt + 1 < KT - 1; kt += 2) {
+        step(int_c<0>{}, int_c<0>{}, kt);
+        step(int_c<1>{}, int_c<0>{}, kt + 1);
+      }
+      if (kt < KT - 1) {
+        step(int_c<0>{}, int_c<0>{}, kt);
+        last_step(int_c<1>{}, kt + 1);
+      } else {
+        last_step(int_c<0>{}, kt);
+      }
+    }
+#endif
   }
 #else
   static_assert(!DIRECT, "DIRECT belongs to the pipelined loop");
