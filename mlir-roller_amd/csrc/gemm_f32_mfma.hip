@@ -27,7 +27,9 @@
 //               barrier that ends a K step; 4 and 5 (DIRECT only) = the same with three and four
 //               LDS buffers, so that loads run two and three K steps ahead of the MFMAs -- for
 //               short K steps whose MFMA time does not cover a trip to HBM
-//   PAD_A,PAD_B extra floats per LDS row of the A tile ([BM][BK+PAD_A]) and B tile ([BK][BN+PAD_B])
+//   PAD_A,PAD_B extra floats per LDS row of the A tile ([BM][BK+PAD_A]) and B tile ([BK][BN+PAD_B]);
+//               LDS holds the A tiles of all buffers first, then the B tiles, so that both tiles of
+//               either buffer are within the 64 KB immediate offset of an LDS read
 //   VEC         4 = 16-byte aligned 128-bit global accesses (needs K%4==0, N%4==0, lda/ldb/ldc%4==0
 //               and 16-byte aligned base pointers), 1 = any K, N, leading dimension and 4-byte
 //               aligned pointers: 128-bit loads at dword alignment with per-element zeroing of
@@ -67,6 +69,10 @@
 //     epilogue the same w accumulators are adjacent in memory again and leave as one vector store.
 // Rows of LDS-A are padded so that (BK+PAD_A)/4 is odd: the 16-byte reads of lanes in consecutive
 // rows then fall into distinct bank groups.
+//
+// The K loop is written for the instruction issue of one wave per SIMD: an LDS read or a global
+// load issues beside the MFMAs for free, an instruction of the vector ALU (an address add, a
+// compare, a select) takes MFMA issue time, and the loop of the aligned 128-bit kernels has none.
 //
 // Summation order is fixed by (BK, MI) alone; there is no split-K and no atomics, so results are
 // bit-identical from run to run.
@@ -261,6 +267,21 @@ DEV __amdgpu_buffer_rsrc_t make_rsrc(const void* base, long bytes) {
   return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, n, 0x00020000);
 }
 
+// Resource of an operand tile for K step kt.  With 128-bit accesses every 16-byte unit is inside the
+// matrix or outside it as a whole and the predicates of the loads decide (an excluded unit gets
+// OOB_OFFSET, which is beyond any range), so the range only has to tell a live tile (everything
+// passes) from one past the end of K (nothing passes): scalar selects, where the exact remainder
+// costs 64-bit compares on the vector unit in every K step.  With dword-aligned rows (VEC == 1) a
+// 128-bit load can straddle the end of the matrix, and the exact range is what zeroes its tail.
+DEV __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, bool live, long bytes) {
+#if VEC == 4
+  (void)bytes;
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, live ? 0x7fffffff : 0, 0x00020000);
+#else
+  return make_rsrc(base, live ? bytes : 0);
+#endif
+}
+
 template <bool SAME = false>
 DEV v4f load_unit(__amdgpu_buffer_rsrc_t r, unsigned off, bool p0, bool p1, bool p2, bool p3) {
 #if VEC == 4
@@ -425,15 +446,15 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   // fills the 64 consecutive 16-byte units that start at unit i*NT + wave*64 of the operand tile.
   // KTAIL (a compile-time 0/1) says whether tile kt may be the one that K ends in: only then are
   // the units tested against K.
-  auto fetch_direct = [&](auto ktail, int kt, int stage) {
+  auto fetch_direct = [&](auto ktail, int kt, int stage) __attribute__((always_inline)) {
     constexpr bool KTEST = EDGE_K && decltype(ktail)::value;
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
     const int k0 = kt * BK;
     const bool live = kt < KT;
-    const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, live ? a_rem - (long)k0 * 4 : 0);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + B_STEP(k0), live ? b_rem - B_STEP(k0) * 4 : 0);
-    float* As = lds + stage * STAGE_FLOATS;
-    float* Bs = As + A_STAGE;
+    const __amdgpu_buffer_rsrc_t ar = tile_rsrc(Ag + k0, live, a_rem - (long)k0 * 4);
+    const __amdgpu_buffer_rsrc_t br = tile_rsrc(Bg + B_STEP(k0), live, b_rem - B_STEP(k0) * 4);
+    float* As = lds + stage * A_STAGE;
+    float* Bs = lds + LDS_BUFS * A_STAGE + stage * B_STAGE;
 #pragma unroll
     for (int i = 0; i < A_PER_T; ++i) {
       const int first = i * NT + wave * 64;
@@ -457,12 +478,12 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   // (the pipelined loop asks for up to two steps ahead) gets an empty resource: every load
   // returns 0 and touches no memory.  KTAIL (a compile-time 0/1) says whether tile kt may be the
   // one that K ends in: only then are the elements tested against K.
-  auto fetch = [&](auto ktail, int kt) {
+  auto fetch = [&](auto ktail, int kt) __attribute__((always_inline)) {
     constexpr bool KTEST = EDGE_K && decltype(ktail)::value;
     const int k0 = kt * BK;
     const bool live = kt < KT;
-    const __amdgpu_buffer_rsrc_t ar = make_rsrc(Ag + k0, live ? a_rem - (long)k0 * 4 : 0);
-    const __amdgpu_buffer_rsrc_t br = make_rsrc(Bg + B_STEP(k0), live ? b_rem - B_STEP(k0) * 4 : 0);
+    const __amdgpu_buffer_rsrc_t ar = tile_rsrc(Ag + k0, live, a_rem - (long)k0 * 4);
+    const __amdgpu_buffer_rsrc_t br = tile_rsrc(Bg + B_STEP(k0), live, b_rem - B_STEP(k0) * 4);
 #pragma unroll
     for (int i = 0; i < A_PER_T; ++i) {
       const int k = k0 + a_kcol[i];
@@ -485,9 +506,9 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     }
   };
 
-  auto stash = [&](int stage) {
-    float* As = lds + stage * STAGE_FLOATS;
-    float* Bs = As + A_STAGE;
+  auto stash = [&](int stage) __attribute__((always_inline)) {
+    float* As = lds + stage * A_STAGE;
+    float* Bs = lds + LDS_BUFS * A_STAGE + stage * B_STAGE;
 #pragma unroll
     for (int i = 0; i < A_PER_T; ++i)
       if (A_UNITS % NT == 0 || tid + i * NT < A_UNITS) *(v4f*)&As[a_soff[i]] = ra[i];
@@ -534,9 +555,9 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     float b1[4];
 #endif
   };
-  auto read_frags = [&](frag_t& f, int stage, int kk) {
-    const float* As = lds + stage * STAGE_FLOATS;
-    const float* Bs = As + A_STAGE;
+  auto read_frags = [&](frag_t& f, int stage, int kk) __attribute__((always_inline)) {
+    const float* As = lds + stage * A_STAGE;
+    const float* Bs = lds + LDS_BUFS * A_STAGE + stage * B_STAGE;
 #pragma unroll
 #if DIRECT
     for (int bi = 0; bi < TM; ++bi) f.a[bi] = *(const v4f*)&As[a_frag + bi * MI * LDA_S + a_round[kk / KSUPER]];
@@ -560,7 +581,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     }
 #endif
   };
-  auto mfma_frags = [&](const frag_t& f, int t0 = 0, int t1 = 4) {
+  auto mfma_frags = [&](const frag_t& f, int t0 = 0, int t1 = 4) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = t0; t < t1; ++t)
 #pragma unroll
@@ -579,34 +600,51 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   // ---- main loop ----
 #if STAGES >= 3
   if (KT > 0) {
-    // Software pipeline.  At the top of step kt: tile kt is in LDS buffer kt&1, its first fragment
+    // Software pipeline.  At the top of step kt: tile kt is in its LDS buffer, its first fragment
     // round is already in registers, and the staging registers hold tile kt+1 (loaded during step
     // kt-1).  Within the step each fragment round is read while the previous one is in the MFMA
     // pipe; before the last round is multiplied, tile kt+1 goes to the other LDS buffer, the
     // loads of tile kt+2 are issued, the workgroup meets at the barrier, and the first fragment
     // round of tile kt+1 is read -- so that the last MFMA group covers that read's latency.
+    //
+    // Instructions of the vector ALU take issue slots from the MFMAs (LDS reads and global loads
+    // do not), so the loop carries none: with two LDS buffers the steps run two per loop trip, the
+    // first of a pair on buffer 0 and the second on buffer 1, both compile-time constants (as is
+    // the fragment set, which alternates too when a step has an odd number of rounds), and every
+    // LDS address is a loop-invariant register plus an immediate offset.  The last step is always
+    // on buffer 0; an odd number of pipelined steps therefore starts with a single step on buffer
+    // 1, and tile 0 goes to buffer `first` = parity of the number of pipelined steps.
     frag_t fr[2];
+    constexpr int ODD = SUPERS % 2;
+    const int pipelined = KT - 1;
+    const int first = pipelined & 1;
 #if DIRECT
 #pragma unroll
-    for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(int_c<1>{}, i, i);
+    for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(int_c<1>{}, i, LDS_BUFS == 2 ? (i ^ first) : i);
     // this wave's part of tile 0 is in LDS (of every requested tile when the loads per wave differ)
     WAIT_VMCNT(PROLOGUE_IN_FLIGHT);
 #else
     fetch(int_c<1>{}, 0);
-    stash(0);
+    stash(first);
     fetch(int_c<1>{}, 1);
 #endif
     __syncthreads();
-    read_frags(fr[0], 0, 0);
+    if (first) {
+      read_frags(fr[ODD], LDS_BUFS == 2 ? 1 : 0, 0);
+    } else {
+      read_frags(fr[0], 0, 0);
+    }
 
     // P = which of the two fragment sets holds round 0 of this step (compile-time, so that the
     // sets stay in fixed registers); the set alternates every round.
     // MFMAs and fragment reads per round; LDS writes and global loads per K step
     constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NSEG), W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
 
-    auto step = [&](auto parity, auto ktail, int kt) {
+    // `buffer`: the LDS buffer of this step's tile when there are two (with more, kt % LDS_BUFS).
+    auto step = [&](auto parity, auto ktail, auto buffer, int kt) __attribute__((always_inline)) {
       constexpr int P = decltype(parity)::value;
-      const int cur = (unsigned)kt % LDS_BUFS, nxt = (unsigned)(kt + 1) % LDS_BUFS;
+      const int cur = LDS_BUFS == 2 ? decltype(buffer)::value : (unsigned)kt % LDS_BUFS;
+      const int nxt = LDS_BUFS == 2 ? 1 - decltype(buffer)::value : (unsigned)(kt + 1) % LDS_BUFS;
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
@@ -659,9 +697,9 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
 #endif
     };
-    auto last_step = [&](auto parity, int kt) {
+    auto last_step = [&](auto parity, auto buffer, int kt) __attribute__((always_inline)) {
       constexpr int P = decltype(parity)::value;
-      const int cur = (unsigned)kt % LDS_BUFS;
+      const int cur = LDS_BUFS == 2 ? decltype(buffer)::value : (unsigned)kt % LDS_BUFS;
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
@@ -677,56 +715,36 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
     };
 
-#if EDGE_K
-    // Pipelined steps [from, to).  An odd number of rounds per step flips the fragment-set parity
-    // every step, so the parity of a step is that of its index.
-    auto steps = [&](auto ktail, int from, int to) {
-      int kt = from;
-      if constexpr (SUPERS % 2 == 0) {
-        for (; kt < to; ++kt) step(int_c<0>{}, ktail, kt);
-      } else {
-        if (kt < to && (kt & 1)) step(int_c<1>{}, ktail, kt++);
-        for (; kt + 1 < to; kt += 2) {
-          step(int_c<0>{}, ktail, kt);
-          step(int_c<1>{}, ktail, kt + 1);
-        }
-        if (kt < to) step(int_c<0>{}, ktail, kt);
-      }
+    // One pair of steps: buffers 0 then 1.
+    // (the scheduling fences keep the interleave directives of one step from picking up the
+    // instructions of the other)
+    auto pair = [&](auto ktail, int kt) __attribute__((always_inline)) {
+      step(int_c<0>{}, ktail, int_c<0>{}, kt);
+      __builtin_amdgcn_sched_barrier(0);
+      step(int_c<ODD>{}, ktail, int_c<1>{}, kt + 1);
+      __builtin_amdgcn_sched_barrier(0);
     };
-    // Step kt requests tile kt + LDS_BUFS.  Only tile KT-1 can be cut short by K, so only the step
-    // that requests it tests its units against K; the steps behind it request tiles past the end
-    // (empty range: zeros whatever the test says) and share its code.
-    const int plain = KT - 1 - LDS_BUFS > 0 ? KT - 1 - LDS_BUFS : 0;
-    steps(int_c<0>{}, 0, plain);
-    steps(int_c<1>{}, plain, KT - 1);
-    if (SUPERS % 2 == 0 || (KT - 1) % 2 == 0) {
-      last_step(int_c<0>{}, KT - 1);
-    } else {
-      last_step(int_c<1>{}, KT - 1);
-    }
-#else
     int kt = 0;
-    if constexpr (SUPERS % 2 == 0) {
-      for (; kt < KT - 1; ++kt) step(int_c<0>{}, int_c<0>{}, kt);
-      last_step(int_c<0>{}, kt);
-    } else {
-      // an odd number of rounds per step flips the parity every step: unroll by two
-      for (; kt + 1 < KT - 1; kt += 2) {
-        step(int_c<0>{}, int_c<0>{}, kt);
-        step(int_c<1>{}, int_c<0>{}, kt + 1);
-      }
-      if (kt < KT - 1) {
-        step(int_c<0>{}, int_c<0>{}, kt);
-        last_step(int_c<1>{}, kt + 1);
-      } else {
-        last_step(int_c<0>{}, kt);
-      }
+    if (first) {
+      // (with a K edge this step may be the one that requests the last tile)
+      step(int_c<ODD>{}, int_c<1>{}, int_c<1>{}, kt);
+      ++kt;
     }
+#if EDGE_K
+    // Step kt requests tile kt + LDS_BUFS.  Only tile KT-1 can be cut short by K, so only the pair
+    // with the step that requests it, and the pairs behind it (they request tiles past the end:
+    // empty range, zeros whatever the test says), test their units against K.
+    const int plain = pipelined - LDS_BUFS;     // steps before the one that requests tile KT-1
+    for (; kt + 1 < plain; kt += 2) pair(int_c<0>{}, kt);
+    for (; kt + 1 < pipelined; kt += 2) pair(int_c<1>{}, kt);
+#else
+    for (; kt + 1 < pipelined; kt += 2) pair(int_c<0>{}, kt);
 #endif
+    last_step(int_c<0>{}, int_c<0>{}, pipelined);
   }
 #else
   static_assert(!DIRECT, "DIRECT belongs to the pipelined loop");
-  auto multiply = [&](int stage) {
+  auto multiply = [&](int stage) __attribute__((always_inline)) {
 #pragma unroll
     for (int kk = 0; kk < BK; kk += KSUPER) {
       frag_t f;
