@@ -334,24 +334,27 @@ class Policy:
 
     def estimate_seconds(self, td: TileDict) -> float:
         """Roofline estimate of the whole GEMM with block tile ``td`` on a device with matrix
-        cores.  The busiest CU works through ceil(grid / CUs) tiles one after another.  A tile
-        costs the larger of its MFMA time at the CU's share of the matrix peak and its traffic at
-        the CU's share of the memory bandwidth.  MFMA time is divided by an issue efficiency that
-        falls with the operand traffic per FLOP, (1/m + 1/n); its two constants are fields of the
-        device model, fitted to a committed sweep (``calibrate.py``).  A fixed cost per tile covers filling the
-        pipeline and draining the accumulators."""
+        cores.  The busiest CU works through ceil(grid / CUs) tiles.  A tile costs the larger of
+        its MFMA time at the CU's share of the matrix peak and its traffic at the CU's share of
+        the memory bandwidth.  MFMA time is divided by an issue efficiency that falls with the
+        operand traffic per FLOP, (1/m + 1/n); its two constants are fields of the device model,
+        fitted to a committed sweep (``calibrate.py``).  A fixed cost per tile covers filling the
+        pipeline and draining the accumulators; workgroups that are resident on a CU together
+        (``block_per_SM``) hide it behind one another's MFMAs, so it is paid once per group of
+        resident tiles."""
         a, cfg = self.arch, self.matmul_config
         m, n = td.block_tile
         cu_flops = a.peak_matrix_tflops * 1e12 / a.compute_max_core
         cu_bw = a.bandwidth[0] * 1e9 / a.compute_max_core
         k_steps = -(-cfg.K // td.rstep)  # the kernel runs whole K steps also where K is ragged
+        tiles_per_cu = -(-td.grid_size // a.compute_max_core)
+        resident = max(1, min(td.block_per_SM, tiles_per_cu))
         base, slope = a.mfma_efficiency
-        efficiency = max(base - slope * (1.0 / m + 1.0 / n), 0.05)
+        efficiency = max(base - slope * (1.0 / m + 1.0 / n) + (a.co_resident_gain if resident > 1 else 0.0), 0.05)
         t_mfma = 2.0 * m * n * k_steps * td.rstep / (cu_flops * efficiency)
         t_mem = td.traffic / cu_bw
         t_fixed = a.tile_fixed_seconds + m * n * cfg.el_bytes / cu_bw
-        tiles_per_cu = -(-td.grid_size // a.compute_max_core)
-        return tiles_per_cu * (max(t_mfma, t_mem) + t_fixed)
+        return tiles_per_cu * max(t_mfma, t_mem) + (-(-tiles_per_cu // resident)) * t_fixed
 
     def get_block_tiles_candidates(self, init_tile: List[int], rstep: int) -> List[TileDict]:
         """All valid block tiles, best first (stable with respect to enumeration order:

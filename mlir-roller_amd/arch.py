@@ -53,8 +53,10 @@ class TileDevice:
     clock_mhz: int = 0
     # ranking model of devices with matrix cores (``Policy.estimate_seconds``): the matrix pipe's
     # issue efficiency on a block tile [m, n] is base - slope * (1/m + 1/n), and every tile pays
-    # ``tile_fixed_seconds`` (pipeline fill) on top of storing its results
+    # ``tile_fixed_seconds`` (pipeline fill) on top of storing its results; workgroups that share a
+    # core fill one another's barrier stalls, which adds ``co_resident_gain`` to the efficiency
     mfma_efficiency: Tuple[float, float] = (1.0, 0.0)
+    co_resident_gain: float = 0.0
     tile_fixed_seconds: float = 0.0
     # wave tiles of at most this many elements list the matrix instruction with the longer k first
     long_k_mfma_up_to: int = 0
@@ -130,7 +132,8 @@ class MI355X(TileDevice):
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
     # (a test refits it): about 0.95 for 256x256 tiles, 0.81 for 32x64
-    mfma_efficiency: Tuple[float, float] = (0.981, 2.07)
+    mfma_efficiency: Tuple[float, float] = (0.999, 2.14)
+    co_resident_gain: float = 0.01
     tile_fixed_seconds: float = 1.0e-6
     # 16x16x4 moves half as many accumulator bytes per FLOP as 32x32x2, which leaves the register
     # file free for LDS fragment reads: it wins on every wave tile it fits (up to 64x128; a wave

@@ -73,14 +73,22 @@ def fixed_tile_seconds(m: int, n: int, arch: TileDevice, el_bytes: int = 4) -> f
     return arch.tile_fixed_seconds + m * n * el_bytes / (arch.bandwidth[0] * 1e9 / arch.compute_max_core)
 
 
+def resident_tiles(rec: dict, arch: TileDevice, depth: int = DEFAULT_PIPELINE_DEPTH) -> int:
+    """Workgroups of this record's block tile that the policy's LDS and register model puts on
+    one CU at a time."""
+    td = TileDict.from_block_tile(list(rec["block_tile"]), rec["rstep"], MatmulConfig(*rec["shape"], 32), arch, depth)
+    return max(1, td.block_per_SM)
+
+
 def observed_efficiency(rec: dict, arch: TileDevice) -> Optional[float]:
     """MFMA issue efficiency that one measurement implies under the model's structure:
-    tiles_per_cu * (ideal / efficiency + fixed) = measured."""
+    tiles_per_cu * ideal / efficiency + ceil(tiles_per_cu / resident) * fixed = measured."""
     M, N, K = rec["shape"]
     m, n = rec["block_tile"]
     tiles = (-(-M // m)) * (-(-N // n))
     per_cu = -(-tiles // arch.compute_max_core)
-    busy = rec["ms"] * 1e-3 / per_cu - fixed_tile_seconds(m, n, arch)
+    rounds = -(-per_cu // min(resident_tiles(rec, arch), per_cu))
+    busy = (rec["ms"] * 1e-3 - rounds * fixed_tile_seconds(m, n, arch)) / per_cu
     if busy <= 0:
         return None
     return ideal_tile_seconds(m, n, K, rec["rstep"], arch) / busy
@@ -97,14 +105,34 @@ def best_per_block_tile(records: Iterable[dict]) -> List[dict]:
     return [best[k] for k in sorted(best)]
 
 
+def _solve(a: List[List[float]], b: List[float]) -> List[float]:
+    """Gaussian elimination with partial pivoting for the small normal equations of ``fit``."""
+    n = len(b)
+    m = [row[:] + [rhs] for row, rhs in zip(a, b)]
+    for col in range(n):
+        piv = max(range(col, n), key=lambda r: abs(m[r][col]))
+        if abs(m[piv][col]) < 1e-18:
+            raise ValueError("the records do not pin the model (singular normal equations)")
+        m[col], m[piv] = m[piv], m[col]
+        for r in range(col + 1, n):
+            f = m[r][col] / m[col][col]
+            for c in range(col, n + 1):
+                m[r][c] -= f * m[col][c]
+    x = [0.0] * n
+    for r in range(n - 1, -1, -1):
+        x[r] = (m[r][n] - math.fsum(m[r][c] * x[c] for c in range(r + 1, n))) / m[r][r]
+    return x
+
+
 def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
-    """Least-squares ``efficiency = base - slope * (1/m + 1/n)`` over the best record of every
-    (shape, block tile) whose tile grid fills at least three quarters of its last round of CUs
-    (a sparse last round measures the tail, not the tile) and that ran for at least ``MIN_FIT_MS``
-    (below that the launch itself is a visible share).  Deterministic: closed-form normal
-    equations, records in sorted order."""
+    """Least-squares ``efficiency = base - slope * (1/m + 1/n) + gain * [tiles share a CU]`` over
+    the best record of every (shape, block tile) whose tile grid fills at least three quarters of
+    its last round of CUs (a sparse last round measures the tail, not the tile) and that ran for at
+    least ``MIN_FIT_MS`` (below that the launch itself is a visible share).  The gain is fitted
+    only when the records hold tiles of both kinds.  Deterministic: closed-form normal equations,
+    records in sorted order."""
     arch = arch or MI355X()
-    xs, ys = [], []
+    xs, ys, zs = [], [], []
     for r in best_per_block_tile(records):
         M, N, _ = r["shape"]
         m, n = r["block_tile"]
@@ -117,16 +145,19 @@ def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
             continue
         xs.append(1.0 / m + 1.0 / n)
         ys.append(eff)
-    if len(xs) < 3:
-        raise ValueError(f"only {len(xs)} usable records; need at least 3 distinct block tiles")
-    n_pts = float(len(xs))
-    sx, sy = math.fsum(xs), math.fsum(ys)
-    sxx, sxy = math.fsum(x * x for x in xs), math.fsum(x * y for x, y in zip(xs, ys))
-    slope = (n_pts * sxy - sx * sy) / (n_pts * sxx - sx * sx)
-    base = (sy - slope * sx) / n_pts
-    resid = [y - (base + slope * x) for x, y in zip(xs, ys)]
-    return {"mfma_efficiency": (round(base, 3), round(-slope, 2)), "base": base, "slope": -slope, "points": len(xs),
-            "rms_residual": math.sqrt(math.fsum(e * e for e in resid) / n_pts)}
+        zs.append(1.0 if min(resident_tiles(r, arch), -(-tiles // arch.compute_max_core)) > 1 else 0.0)
+    if len(set(xs)) < 3:
+        raise ValueError(f"only {len(set(xs))} usable block-tile sizes; need at least 3")
+    with_gain = 0.0 < math.fsum(zs) < len(zs)
+    cols = [[1.0] * len(xs), xs] + ([zs] if with_gain else [])
+    normal = [[math.fsum(p * q for p, q in zip(ci, cj)) for cj in cols] for ci in cols]
+    rhs = [math.fsum(p * y for p, y in zip(ci, ys)) for ci in cols]
+    sol = _solve(normal, rhs)
+    base, slope, gain = sol[0], -sol[1], (sol[2] if with_gain else 0.0)
+    resid = [y - (base - slope * x + gain * z) for x, y, z in zip(xs, ys, zs)]
+    return {"mfma_efficiency": (round(base, 3), round(slope, 2)), "co_resident_gain": round(gain, 3), "base": base,
+            "slope": slope, "gain": gain, "points": len(xs),
+            "rms_residual": math.sqrt(math.fsum(e * e for e in resid) / len(xs))}
 
 
 def _geo_mean(ratios: Sequence[float]) -> float:
@@ -318,8 +349,8 @@ def main(argv=None) -> int:
     if args.cmd == "fit":
         res = fit(data["records"])
         now = MI355X()
-        print(f"fitted mfma_efficiency = {res['mfma_efficiency']} from {res['points']} block tiles "
-              f"(rms residual {res['rms_residual']:.4f}); arch.MI355X has {tuple(now.mfma_efficiency)}")
+        print(f"fitted mfma_efficiency = {res['mfma_efficiency']}, co_resident_gain = {res['co_resident_gain']} from {res['points']} "
+              f"block tiles (rms residual {res['rms_residual']:.4f}); arch.MI355X has {tuple(now.mfma_efficiency)}, {now.co_resident_gain}")
         waves = fit_waves_per_simd(data["records"])
         print(f"fitted waves_per_partition = {waves['waves_per_partition']} (two waves per SIMD take {waves['two_over_one']:.4f} x "
               f"the time of one, {waves['pairs']} block tiles); arch.MI355X has {now.waves_per_partition}")
