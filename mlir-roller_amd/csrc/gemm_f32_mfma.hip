@@ -278,7 +278,13 @@ DEV __amdgpu_buffer_rsrc_t tile_rsrc(const void* base, bool live, long bytes) {
   (void)bytes;
   return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, live ? 0x7fffffff : 0, 0x00020000);
 #else
-  return make_rsrc(base, live ? bytes : 0);
+  // a live tile has a positive remainder; "above 2^31-1" as a test for set upper bits stays on
+  // the scalar unit, where an ordered 64-bit compare would go to the vector unit
+  unsigned hi = (unsigned)((unsigned long)bytes >> 32);
+  const unsigned lo = (unsigned)bytes;
+  asm("" : "+s"(hi));   // (keeps the halves apart: put back together, the test is a 64-bit compare)
+  const int n = (hi | (lo >> 31)) != 0 ? 0x7fffffff : (int)lo;
+  return __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, live ? n : 0, 0x00020000);
 #endif
 }
 
@@ -499,9 +505,11 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
                                 b_ok[i][0] && (!KTEST || k + 0 < K), b_ok[i][1] && (!KTEST || k + 1 < K),
                                 b_ok[i][2] && (!KTEST || k + 2 < K), b_ok[i][3] && (!KTEST || k + 3 < K));
 #else
+      // Columns at or beyond N only ever meet columns of C that are not stored, so a unit that
+      // straddles N needs no zeroing: it is loaded if its first column is inside (what lies
+      // past the end of the last row of B is beyond the range and comes back as zero).
       const bool kin = !KTEST || k0 + b_krow[i] < K;
-      rb[i] = load_unit<!EDGE>(br, b_goff[i], b_ok[i][0] && kin, b_ok[i][1] && kin, b_ok[i][2] && kin,
-                               b_ok[i][3] && kin);
+      rb[i] = load_unit<true>(br, b_goff[i], b_ok[i][0] && kin, false, false, false);
 #endif
     }
   };
