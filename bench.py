@@ -108,10 +108,18 @@ extern "C" __global__ __launch_bounds__(256) void clock_probe(long long* out, fl
 
 
 # Engine clock under the GEMM load itself: one wave on a second stream sleeps and samples the two
-# counters while the timed steps run; it ends after `ticks` of the 100 MHz counter or `max_iters`
-# samples, whichever comes first.
+# counters while the timed steps run.  It starts sampling when `flag` is raised (a one-thread kernel
+# queued on the GEMM stream right ahead of the timed region does that; the wait gives up after
+# `max_wait` naps) and ends after `ticks` of the 100 MHz counter or `max_iters` samples, whichever
+# comes first.
 SAMPLER_KERNEL = r"""
-extern "C" __global__ void clock_sampler(long long* out, long long ticks, int max_iters) {
+extern "C" __global__ void raise_flag(long long* flag) { __hip_atomic_store(flag, 1LL, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT); }
+extern "C" __global__ void clock_sampler(long long* out, long long* flag, long long ticks, int max_wait, int max_iters) {
+  int waited = 0;
+  while (__hip_atomic_load(flag, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) == 0 && waited < max_wait) {
+    __builtin_amdgcn_s_sleep(127);
+    ++waited;
+  }
   const long long r0 = __builtin_amdgcn_s_memrealtime();
   const long long c0 = __builtin_readcyclecounter();
   long long r = r0, c = c0;
@@ -122,7 +130,7 @@ extern "C" __global__ void clock_sampler(long long* out, long long ticks, int ma
     c = __builtin_readcyclecounter();
     ++it;
   }
-  if (threadIdx.x == 0) { out[0] = c - c0; out[1] = r - r0; out[2] = it; }
+  if (threadIdx.x == 0) { out[0] = c - c0; out[1] = r - r0; out[2] = it; out[3] = waited; }
 }
 """
 
@@ -396,7 +404,9 @@ def main() -> int:
         probe_out, probe_sink = DeviceArray((2 * probe_waves,), np.int64), DeviceArray((probe_waves,))
         sampler_mod = Module(hip.compile_source(SAMPLER_KERNEL, "clock_sampler.hip")[0])
         clock_sampler = sampler_mod.get_function("clock_sampler")
+        raise_flag = sampler_mod.get_function("raise_flag")
         sampler_out = DeviceArray.zeros((4,), np.int64)
+        sampler_flag = DeviceArray.zeros((1,), np.int64)
         side_stream = Stream()
         # sample for about 70 % of what the timed steps should take (tuned times; 1 ms at least)
         expect_ms = args.steps * sum(c["tuned_ms"] if c["tuned_ms"] == c["tuned_ms"] else 2.0 * c["shape"][0] * c["shape"][1] * c["shape"][2] / 120e9
@@ -408,9 +418,12 @@ def main() -> int:
         one_step()
     e0, e1 = Event(), Event()
     wall0 = time.perf_counter()
-    e0.record(stream)
     if clock_probe is not None:
-        clock_sampler((1,), (64,), (sampler_out, ctypes.c_longlong(sampler_ticks), max(1000, sampler_ticks // 20)), stream=side_stream)
+        # (the sampler naps about 3.4 us at a time: 200 000 naps outlast any warm-up that fits this script)
+        clock_sampler((1,), (64,), (sampler_out, sampler_flag, ctypes.c_longlong(sampler_ticks), 200000, max(1000, sampler_ticks // 20)),
+                      stream=side_stream)
+        raise_flag((1,), (1,), (sampler_flag,), stream=stream)
+    e0.record(stream)
     for _ in range(args.steps):
         one_step()
     e1.record(stream)
@@ -427,7 +440,7 @@ def main() -> int:
     if clock_probe is not None:
         ticks = probe_out.get().reshape(-1, 2).astype(np.float64)
         probe_mhz = round(float(np.median(ticks[:, 0] / np.maximum(ticks[:, 1], 1.0))) * 100.0, 1)
-        cycles, real, _samples, _ = (int(v) for v in sampler_out.get())
+        cycles, real, _samples, _naps = (int(v) for v in sampler_out.get())
         if real > 0:
             achieved_mhz = round(cycles / real * 100.0, 1)
             sampler_ms = round(real / 1e5, 3)
