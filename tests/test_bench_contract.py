@@ -59,6 +59,8 @@ def test_clock_kernels_compile_for_gfx950(hip_lib):
     for source, symbol in ((bench.CLOCK_KERNEL, b"clock_probe"), (bench.SAMPLER_KERNEL, b"clock_sampler"), (bench.COPY_KERNEL, b"copy_kernel")):
         code, _ = hip.compile_source(source, "k.hip")
         assert code[:4] == b"\x7fELF" and symbol in code
+    # the sampler starts on a flag that a second kernel of the same module raises
+    assert b"raise_flag" in hip.compile_source(bench.SAMPLER_KERNEL, "k.hip")[0]
 
 
 def test_named_configurations_are_the_four_of_the_baseline():
