@@ -184,19 +184,26 @@ def measured_traffic(workload: str, kernels: dict):
         table = json.loads(TRAFFIC_FILE.read_text())
     except Exception:
         return None, f"{TRAFFIC_FILE.name} not found"
-    entry = table.get(workload)
-    if not entry and set(kernels) <= set(table.get("sweep", {}).get("per_shape", {})):
-        entry = table["sweep"]   # a single shape of the sweep: its row of the sweep's counter run
-    if not entry:
+    # counter runs that cover these shapes: the workload's own and, for shapes of the sweep, the sweep's
+    entries = [table[w] for w in (workload, "sweep") if w in table and set(kernels) <= set(table[w].get("per_shape", {}))]
+    if not entries:
         return None, f"no counter run recorded for workload {workload!r}"
-    per_shape = entry.get("per_shape", {})
-    differing = sorted(k for k, tag in kernels.items()
-                       if k not in per_shape or traffic_key(per_shape[k]["kernel"]) != traffic_key(tag))
+    total, differing = 0.0, []
+    for name, tag in kernels.items():
+        measured = []
+        for entry in entries:
+            measured.append(entry["per_shape"][name])
+            measured += entry.get("other_kernels", {}).get(name, [])   # the same workload run with other kernels kept
+        hit = [m for m in measured if traffic_key(m["kernel"]) == traffic_key(tag)]
+        if hit:
+            total += hit[0]["traffic_bytes"]
+        else:
+            differing.append(name)
     if differing:
+        differing.sort()
         return None, ("counter run was taken with other block tiles for " + ", ".join(differing[:4])
                       + ("..." if len(differing) > 4 else ""))
-    total = sum(per_shape[k]["traffic_bytes"] for k in kernels)
-    return float(total) / len(kernels), entry.get("source", "")
+    return total / len(kernels), entries[0].get("source", "")
 
 
 def main() -> int:
