@@ -670,6 +670,10 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #if SCHED
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
+      // the barrier (and the wait for the LDS reads that comes with it) stays behind the MFMAs above:
+      // left to float, it lands right behind the last read and the wave sits out that read's latency
+      interleave_with_mfma<G / 4, 0, 0x100>();
+      __builtin_amdgcn_sched_barrier(0);
 #endif
       WAIT_VMCNT((LDS_BUFS - 2) * LOADS_PER_TILE);
       __syncthreads();
