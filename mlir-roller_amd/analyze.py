@@ -379,8 +379,10 @@ class Policy:
     def _expand_reduce_axis(self, td: TileDict) -> None:
         """Grows ``td.rstep`` to the multiple of the base step that gives the longest contiguous
         operand rows while one stage still fits the block's share of workgroup memory (the
-        share among the blocks a core actually hosts, when matrix cores are modelled).  Only
-        ``rstep`` and ``smem_cost`` change; occupancy figures keep their base-step values."""
+        share among the blocks a core actually hosts, when matrix cores are modelled) -- or, on
+        a device whose model says not to grow it, takes the shortest such step (among those that
+        let the loads go straight to LDS, if any does).  Only ``rstep`` and ``smem_cost``
+        change; occupancy figures keep their base-step values."""
         resident = td.block_per_SM
         if self.arch.has_matrix_cores:
             # a grid that does not fill the device leaves each core fewer blocks to host
@@ -394,7 +396,10 @@ class Policy:
             # a step that lets the loads go straight to LDS beats a longer one that does not
             direct = [s for s in steps if loads_go_direct_to_lds(self.matmul_config, td.block_tile, s, self.pipeline_depth)]
             steps = direct or steps
-        td.rstep = max(steps, key=lambda s: self._coalesced_score(td.block_tile, s, "raw"))
+        if self.arch.grow_reduce_step:
+            td.rstep = max(steps, key=lambda s: self._coalesced_score(td.block_tile, s, "raw"))
+        else:
+            td.rstep = min(steps)
         td.smem_cost = td.infer_smem_usage()
 
     # ---- threads per block --------------------------------------------------------------------

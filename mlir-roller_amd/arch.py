@@ -60,6 +60,10 @@ class TileDevice:
     tile_fixed_seconds: float = 0.0
     # wave tiles of at most this many elements list the matrix instruction with the longer k first
     long_k_mfma_up_to: int = 0
+    # whether the reduce step of a tile grows to what its share of workgroup memory allows (longer
+    # contiguous rows, fewer loop trips: the reference's rule) or stays at the shortest step that
+    # suits the loads (smaller stages, more blocks resident on a core)
+    grow_reduce_step: bool = True
 
     def get_avaliable_tensorintrin_shapes(self) -> List[Tuple[int, int, int]]:
         """Matrix-instruction shapes of the device (name kept from the reference, arch.py:36)."""
@@ -132,13 +136,17 @@ class MI355X(TileDevice):
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
     # (a test refits it): about 0.95 for 256x256 tiles, 0.81 for 32x64
-    mfma_efficiency: Tuple[float, float] = (0.999, 2.14)
-    co_resident_gain: float = 0.01
+    mfma_efficiency: Tuple[float, float] = (0.988, 0.92)
+    co_resident_gain: float = 0.008
     tile_fixed_seconds: float = 1.0e-6
     # 16x16x4 moves half as many accumulator bytes per FLOP as 32x32x2, which leaves the register
     # file free for LDS fragment reads: it wins on every wave tile it fits (up to 64x128; a wave
     # keeps at most 32 blocks), by 0.3-1 % in the committed sweep
     long_k_mfma_up_to: int = 64 * 128
+    # a 32-wide K step already reads whole 128-byte lines; a longer one only takes the LDS that a
+    # second workgroup on the CU would use and lengthens the fill of the pipeline (measured: 128x128
+    # tiles at K steps of 32 against 64, 64x64 at 32 / 64 / 128: the shortest wins or ties)
+    grow_reduce_step: bool = False
     smem_cap: int = field(init=False)
     max_smem_usage: int = field(init=False)
 

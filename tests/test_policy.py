@@ -289,13 +289,16 @@ def test_mi355x_block_sizes_aim_for_one_wave_per_simd():
     assert policy.score_block_size(192) > policy.score_block_size(512)  # three waves leave a SIMD idle
     assert Policy(cfg, CUDA()).recommend_block_size(TileDict.from_block_tile([128, 128], 32, cfg, CUDA()))[0] == 128
     hints = get_roller_hints(cfg, MI355X(), topk=4)
-    # one block tile at two block sizes, then the next tile.  The 16x16x4 shape is out for 256x256:
-    # at four waves 128x128 would be 64 blocks, more than the kernel keeps in registers, and at eight
-    # waves 4 x 8 blocks of 16x16 need more fragment registers than half a SIMD's file leaves.  Next
-    # comes the tile of which two fit a CU at once (each hides the other's barriers, fill and drain)
+    # one block tile at two block sizes, then the next tile.  First the tile of which two fit a CU
+    # at once (each hides the other's barriers, fill and drain), with the 16x16x4 instruction
     assert [(h.block_tile, h.wave_tile, h.threads, h.mfma) for h in hints] == [
-        ([256, 256], [128, 128], 256, 32), ([256, 256], [64, 128], 512, 32),
-        ([128, 128], [64, 64], 256, 16), ([128, 128], [32, 64], 512, 16)]
+        ([128, 128], [64, 64], 256, 16), ([128, 128], [32, 64], 512, 16),
+        ([64, 256], [64, 64], 256, 16), ([64, 256], [32, 64], 512, 16)]
+    # 256x256 (one per CU) is out for 16x16x4: at four waves 128x128 would be 64 blocks, more than the
+    # kernel keeps in registers, and at eight waves 4 x 8 blocks of 16x16 need more fragment registers
+    # than half a SIMD's file leaves
+    big = [h for h in get_roller_hints(cfg, MI355X(), topk=40) if h.block_tile == [256, 256]]
+    assert [(h.wave_tile, h.threads, h.mfma) for h in big] == [([128, 128], 256, 32), ([64, 128], 512, 32)]
     assert analyze.split_block_over_waves([256, 256], 4, 32, MI355X(), shapes=[(16, 16, 4)]) is None
     assert analyze.split_block_over_waves([256, 128], 4, 32, MI355X(), shapes=[(16, 16, 4)]) == ([64, 128], 16)   # 4 x 8 = 32 blocks
 
@@ -320,16 +323,26 @@ def test_mi355x_register_budget_drops_splits_that_would_spill():
     assert policy._assign_wave_tiles(td, 96) == []                                 # not a whole number of waves
 
 
-def test_mi355x_reduce_step_grows_when_the_grid_leaves_room():
+def test_mi355x_reduce_step_stays_short_unless_the_device_model_says_grow():
+    import dataclasses
     arch = MI355X()
-    # 2048^2 output, 128x128 tiles: 256 blocks on 256 CUs -> one block per CU -> the whole 80 KB stage budget
+    assert not arch.grow_reduce_step and CUDA().grow_reduce_step
+    # the committed model: every hint keeps the 32-wide step (whole 128-byte lines, smallest stages)
+    for shape in SHAPES_MI:
+        assert {h.rstep for h in get_roller_hints(MatmulConfig(*shape, 32), arch, topk=8)} == {32}, shape
     small = [h for h in get_roller_hints(MatmulConfig(2048, 2048, 2048, 32), arch, topk=8) if h.block_tile == [128, 128]][0]
-    assert (small.rstep, small.smem_cost, small.block_per_SM) == (64, 65536, 2)
+    assert (small.rstep, small.smem_cost, small.block_per_SM) == (32, 32768, 2)
+    # with growth switched on (the reference's rule) the step takes the share of LDS a block really has:
+    # 2048^2 output, 128x128 tiles: 256 blocks on 256 CUs -> one block per CU -> the whole 80 KB stage budget
+    grow = dataclasses.replace(arch, grow_reduce_step=True)
+    cfg = MatmulConfig(2048, 2048, 2048, 32)
+    td = TileDict.from_block_tile([128, 128], 32, cfg, grow)
+    Policy(cfg, grow)._expand_reduce_axis(td)
+    assert (td.rstep, td.smem_cost) == (64, 65536)
     # 4096x8192 output with the same tile: 8 blocks per CU, two resident -> 40 KB each -> step stays 32
     cfg = MatmulConfig(4096, 8192, 4096, 32)
-    policy = Policy(cfg, arch)
-    td = TileDict.from_block_tile([128, 128], 32, cfg, arch)
-    policy._expand_reduce_axis(td)
+    td = TileDict.from_block_tile([128, 128], 32, cfg, grow)
+    Policy(cfg, grow)._expand_reduce_axis(td)
     assert td.rstep == 32
 
 
@@ -358,8 +371,8 @@ def test_mi355x_small_wave_tiles_list_the_long_k_instruction_first():
     first = lambda shape: get_roller_hints(MatmulConfig(*shape, 32), arch, topk=2)
     a, b = first((2048, 2048, 2048))                       # 64x128 over four, then eight waves
     assert (a.block_tile, a.wave_tile, a.mfma, b.wave_tile, b.mfma) == ([64, 128], [32, 64], 16, [32, 32], 16)
-    a, b = first((4096, 8192, 4096))                       # 128x128 wave tiles do not fit 16x16x4 (64 blocks)
-    assert a.mfma == 32 and b.mfma == 32 and a.wave_tile == [128, 128]
+    a, b = first((4096, 8192, 4096))                       # 128x128 over four, then eight waves
+    assert (a.block_tile, a.wave_tile, a.mfma, b.wave_tile, b.mfma) == ([128, 128], [64, 64], 16, [32, 64], 16)
     both = Policy(MatmulConfig(2048, 4096, 2048, 32), arch)._assign_wave_tiles(
         TileDict.from_block_tile([128, 256], 32, MatmulConfig(2048, 4096, 2048, 32), arch), 256)
     assert [(t.wave_tile, t.mfma) for t in both] == [([64, 128], 16), ([64, 128], 32)]   # up to 64x128: long k first
@@ -368,8 +381,8 @@ def test_mi355x_small_wave_tiles_list_the_long_k_instruction_first():
 def test_committed_ranking_constants_equal_a_refit_of_the_committed_sweep():
     """The MI355X ranking model is reproducible from the tree: refitting the committed sweep gives
     the constants that ``arch.MI355X`` carries, and replaying the policy on that sweep finds a kernel
-    within one percent of the fastest measured one among its first four hints (and already with its
-    first hint) on every benchmark shape."""
+    within one percent of the fastest measured one among its first four hints (one and a half
+    percent with its first hint alone) on every benchmark shape."""
     from mlir_roller_amd import calibrate
     data = calibrate.load()
     records = data["records"]
@@ -386,7 +399,7 @@ def test_committed_ranking_constants_equal_a_refit_of_the_committed_sweep():
     for shape in list(README_SHAPES) + [(3000, 5000, 1536)]:
         row = rows[shape]
         assert row["unmeasured_in_topk"] == 0 and row["topk_over_fastest"] <= 1.01, row
-        assert row["top1_over_fastest"] <= 1.01, row
+        assert row["top1_over_fastest"] <= 1.015, row
 
 
 def test_refit_rejects_a_sweep_that_cannot_pin_the_model():
