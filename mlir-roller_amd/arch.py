@@ -124,9 +124,10 @@ class MI355X(TileDevice):
     # the kernel's register-staged path pads every row of the LDS A tile by one 16-byte unit; its
     # direct-to-LDS path (K, N multiples of 4 and a power-of-two reduce step) swizzles instead
     lds_row_pad: int = 4
-    # waves per SIMD that the block-size recommendation tries first.  With loads going straight to
-    # LDS one wave per SIMD is enough to keep the matrix pipe fed, and its larger wave tile reads
-    # fewer operand bytes per FLOP (fitted to the committed sweep, see ``calibrate.py``)
+    # waves per SIMD that the block-size recommendation tries first: one per workgroup (fitted to
+    # the committed sweep, see ``calibrate.py``: a workgroup of eight waves takes 1.003 x the time of
+    # one of four on the same block tile); further waves on a SIMD come from other workgroups
+    # that are resident on the CU at the same time
     waves_per_partition: int = 1
     # 256 architectural + 256 accumulation registers per lane, shared by the waves of a SIMD
     regs_per_lane: int = 512
@@ -135,13 +136,13 @@ class MI355X(TileDevice):
     peak_matrix_tflops: float = 157.3
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
-    # (a test refits it): about 0.95 for 256x256 tiles, 0.81 for 32x64
+    # (a test refits both): 0.981 for 256x256 tiles, 0.974 + 0.008 for 128x128 with two on a CU,
+    # 0.945 for 32x64
     mfma_efficiency: Tuple[float, float] = (0.988, 0.92)
     co_resident_gain: float = 0.008
     tile_fixed_seconds: float = 1.0e-6
-    # 16x16x4 moves half as many accumulator bytes per FLOP as 32x32x2, which leaves the register
-    # file free for LDS fragment reads: it wins on every wave tile it fits (up to 64x128; a wave
-    # keeps at most 32 blocks), by 0.3-1 % in the committed sweep
+    # 16x16x4 wins on every wave tile it fits (up to 64x128; a wave keeps at most 32 blocks), by
+    # 0.5-2 % in the committed sweep
     long_k_mfma_up_to: int = 64 * 128
     # a 32-wide K step already reads whole 128-byte lines; a longer one only takes the LDS that a
     # second workgroup on the CU would use and lengthens the fill of the pipeline (measured: 128x128
