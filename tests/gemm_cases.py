@@ -30,7 +30,10 @@ def seeded_policy_cases(arch, count: int = 40, seed: int = 20240607):
         yield case, config, hints[int(rng.integers(0, len(hints)))], depth, trans_b, accumulate
 
 
-def seeded_template_cases(count: int = 72, seed: int = 20250101):
+TEMPLATE_SEEDS = (20250101, 11)
+
+
+def seeded_template_cases(count: int = 72, seed: int = TEMPLATE_SEEDS[0]):
     """Yields ``(case, GemmConfig, (M, N, K))``: random points of the kernel template's own
     parameter space -- not what the policy would pick -- with a problem size to match: both matrix
     instructions, 1 to 8 waves, 1 to 7 column blocks per wave, K steps of 1 to 8 fragment rounds,
