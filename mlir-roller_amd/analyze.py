@@ -111,6 +111,19 @@ def loads_go_direct_to_lds(matmul_config: "MatmulConfig", block_tile: Sequence[i
             and rstep & (rstep - 1) == 0 and (m * rstep // 4) % 64 == 0 and (rstep * n // 4) % 64 == 0)
 
 
+def lds_row_pad(rstep: int, mfma: int) -> int:
+    """Floats of padding per row of a K-contiguous LDS tile ([rows][rstep + pad]) on the MFMA kernel's
+    register-staged path, chosen so that the 128-bit fragment reads touch every bank once per LDS
+    cycle.  With the 32x32x2 instruction a lane group is 32 rows at one k offset: an odd number of
+    16-byte units per row does it.  With 16x16x4 the LDS serves quarter-waves of two lane groups (one
+    unit apart in k) in the same cycle, and rows of 2 mod 4 units keep them apart (measured with a
+    single-wave probe under the profiler: rows of 9 units conflict, rows of 10 do not)."""
+    units = rstep // 4
+    if mfma == 16:
+        return (2 - units) % 4 * 4
+    return 0 if units % 2 else 4
+
+
 def _natural_size(nbytes: float) -> str:
     """1536 -> '1.5 KiB' (binary units, one decimal)."""
     if abs(nbytes) < 1024:
@@ -175,11 +188,11 @@ class TileDict:
         step = self.rstep if rstep is None else rstep
         cfg = self.matmul_config
         # The MFMA kernel keeps the [m, rstep] tile unpadded only on its direct-to-LDS path;
-        # otherwise every row grows by ``lds_row_pad`` wherever that keeps its 128-bit reads
-        # conflict-free (an even number of 16-byte units per row).
-        pad = self.lds_row_pad
-        if not pad or (step // 4) % 2 or loads_go_direct_to_lds(cfg, self.block_tile, step, self.pipeline_depth):
-            pad = 0
+        # otherwise every row is padded to keep its 128-bit reads conflict-free (by how much depends
+        # on the matrix instruction; before one is assigned, the 32x32x2 figure stands in).
+        pad = 0
+        if self.lds_row_pad and not loads_go_direct_to_lds(cfg, self.block_tile, step, self.pipeline_depth):
+            pad = lds_row_pad(step, self.mfma or 32)
         return (step * sum(self.block_tile) + pad * self.block_tile[0]) * cfg.el_bytes
 
     @classmethod
@@ -499,11 +512,16 @@ class Policy:
                 continue
             if budget and acc_regs + self._reg_overhead(td, wave_tile, mi, block_size) > budget:
                 continue
-            td.thread_tile = thread_tile
-            td.wave_tile = wave_tile
-            td.mfma = mi
-            td.threads = block_size
-            out.append(td.clone())
+            done = td.clone()
+            done.thread_tile = thread_tile
+            done.wave_tile = wave_tile
+            done.mfma = mi
+            done.threads = block_size
+            done.smem_cost = done.infer_smem_usage()   # the row padding follows the instruction
+            if done.smem_cost > arch.smem_cap:
+                continue
+            td.thread_tile, td.wave_tile, td.mfma, td.threads = thread_tile, wave_tile, mi, block_size
+            out.append(done)
         # The instruction with the longer k (16x16x4) moves half as many accumulator bytes per FLOP,
         # which leaves the register file free for LDS fragment reads; up to the wave-tile size the
         # device model names it is listed first.

@@ -176,6 +176,16 @@
 #define CPR (BK / 4)
 #define RPL (CPR >= 16 ? 1 : 16 / CPR)
 #define SWZ_N (CPR >= 16 ? 16 : CPR)
+/* The LDS serves a 32-bit read 32 lanes a cycle (lanes 0-31, then 32-63) out of 32 banks.  With the
+ * 16x16x4 instruction the two lane groups of a cycle read rows 4 apart, and a row is a multiple of 32
+ * floats from the next one that matters, so the lone column block of a wave (TN odd: 16 consecutive
+ * floats per lane group) would come from the same 16 banks for both groups.  On rows whose k group
+ * (k / 4) is odd, the waves 2j and 2j+1 along N therefore swap their lone blocks' columns in LDS: the
+ * two are WN = 16 * odd floats apart, i.e. 16 banks, so the groups of a cycle read disjoint banks.
+ * The 128-bit reads keep their columns: the LDS pairs quarter-waves of different lane groups in one
+ * cycle and needs all lane groups on the same bank alignment there.  Needs an even number of waves
+ * along N; the loader fetches the global columns that belong in its LDS slot. */
+#define LONE_SWAP (!TRANS_B && MI == 16 && (TN % 2) == 1 && (NWN % 2) == 0)
 
 static_assert(MI == 32 || MI == 16, "MI selects v_mfma_f32_32x32x2_f32 or v_mfma_f32_16x16x4_f32");
 static_assert(BM % WM == 0 && BN % WN == 0, "wave tile must divide block tile");
@@ -321,6 +331,15 @@ DEV int bt_col_of_row(int row) {
 }
 #endif
 
+// Tile column that sits at float column `col` of LDS row `krow` of the B[K,N] tile (an involution).
+DEV constexpr int b_tile_col(int krow, int col) {
+#if LONE_SWAP
+  if (((krow >> 2) & 1) && col % WN >= (TN - 1) * MI) return ((col / WN) ^ 1) * WN + col % WN;
+#endif
+  (void)krow;
+  return col;
+}
+
 // The same with STRIDE MFMAs ahead of each of the NO other instructions (needs NO * STRIDE <= NM).
 template <int NM, int NO, int MASK, int STRIDE>
 DEV void stride_with_mfma() {
@@ -420,9 +439,10 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
     for (int e = 0; e < 4; ++e) b_ok[i][e] = in && (!EDGE || n0 + col < N);
 #else
-    const int krow = u / (BN / 4), c = u % (BN / 4);
+    // LDS unit u sits in row krow of the tile at float column 4 * slot and holds tile column 4 * c
+    const int krow = u / (BN / 4), slot = u % (BN / 4), c = b_tile_col(krow, slot * 4) / 4;
     b_goff[i] = (unsigned)(krow * ldb + c * 4) * 4u;
-    b_soff[i] = krow * LDB_S + c * 4;
+    b_soff[i] = krow * LDB_S + slot * 4;
     b_krow[i] = krow;
 #pragma unroll
     for (int e = 0; e < 4; ++e) b_ok[i][e] = in && (!EDGE || n0 + c * 4 + e < N);
@@ -548,6 +568,8 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   const int b_frag = (wn0 + lr) * LDB_S + 4 * lg;       // + bj*MI*LDB_S + kk
 #else
   const int b_frag = (4 * lg) * LDB_S + wn0;            // + (kk+t)*LDB_S + b0*MI + w*lr per segment
+  // LONE_SWAP: lanes of an odd k group find their wave's lone column block where the partner wave's is
+  const int b_frag_lone = (4 * lg) * LDB_S + ((LONE_SWAP && (lg & 1)) ? (((wave % NWN) ^ 1) * WN) : wn0) + (TN - 1) * MI + lr;
 #endif
 
   // One round of LDS fragment reads: TM 128-bit reads of A (four consecutive k each) and, for each
@@ -585,7 +607,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
       for (int v = 0; v < NSEG4; ++v) f.b4[t][v] = *(const v4f*)&row[4 * v * MI + 4 * lr];
       if constexpr (HAS_SEG2) f.b2[t] = *(const v2f*)&row[4 * NSEG4 * MI + 2 * lr];
-      if constexpr (HAS_SEG1) f.b1[t] = row[(TN - 1) * MI + lr];
+      if constexpr (HAS_SEG1) f.b1[t] = Bs[b_frag_lone + (kk + t) * LDB_S];
     }
 #endif
   };

@@ -22,7 +22,7 @@ from typing import Optional, Tuple
 import numpy as np
 
 from . import hip
-from .analyze import MatmulConfig, TileDict, get_roller_hints, loads_go_direct_to_lds, split_block_over_waves
+from .analyze import MatmulConfig, TileDict, get_roller_hints, lds_row_pad, loads_go_direct_to_lds, split_block_over_waves
 from .arch import MI355X
 from .hip import DeviceArray, Event, GemmConfig, GemmPlan
 from .utils import get_block_dims
@@ -78,8 +78,8 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
     # whenever both operand tiles are whole waves of 16-byte units and the K step is a power of
     # two (the swizzle is an XOR).
     direct = int(loads_go_direct_to_lds(config, (bm, bn), bk, stages))
-    # otherwise (bk + pad)/4 odd keeps the 128-bit reads of LDS-A free of bank conflicts
-    pad_a = 0 if direct else (4 if (bk // 4) % 2 == 0 else 0)
+    # otherwise padded rows keep the 128-bit reads of LDS-A free of bank conflicts
+    pad_a = 0 if direct else lds_row_pad(bk, mi)
     # a transposed second operand sits in LDS like A and wants the same padding
     pad_b = pad_a if trans_b else 0
     # Padding is an optimisation, fitting the CU is not: a hint whose policy ran for another depth

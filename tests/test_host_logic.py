@@ -33,7 +33,7 @@ def test_direct_path_needs_a_power_of_two_k_step():
     hint = get_roller_hints(cfg, MI355X(), 1)[0].clone()
     hint.rstep = 48
     g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3)
-    assert (g.bk, g.direct, g.pad_a) == (48, 0, 4)
+    assert (g.bk, g.direct, g.mi, g.pad_a) == (48, 0, 16, 8)      # 16x16x4: rows of 2 mod 4 sixteen-byte units
     hint.rstep = 64
     assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).direct == 1
 
@@ -44,7 +44,7 @@ def test_hint_to_gemm_config_ragged_problem():
     assert g.edge == 2 and g.vec == 4 and 1536 % g.bk == 0   # 5000 and 1536 are multiples of 4; K is a whole number of steps
     cfg = MatmulConfig(37, 53, 29, 32)
     g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0], pipeline_depth=3)
-    assert g.edge == 1 and g.vec == 1 and g.direct == 0 and g.pad_a == 4   # dword path keeps padded rows
+    assert g.edge == 1 and g.vec == 1 and g.direct == 0 and (g.mi, g.pad_a) == (16, 8)   # dword path keeps padded rows
 
 
 def test_hint_from_the_a100_model_still_maps_to_wave_tiles():
