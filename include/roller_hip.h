@@ -79,7 +79,34 @@ typedef struct rl_gemm_config {
   int trans_b;     /* 1: the second operand is Bt[N][ldb>=K], C = A*Bt^T (the [spatial, reduce]
                       layout of MatmulConfig.get_input_shapes, src/analyze.py:33-41); pad_b then
                       pads the K-contiguous rows of its LDS tile like pad_a                   */
+  int streamk;     /* 0: one workgroup per tile of C, grid (ceil(N/bn), ceil(M/bm)) as at src/roller.py:536.
+                      1..8: a fixed grid of that many workgroups per CU; each works an equal share of all
+                      (tile, K step) units, tiles whose K range is split are summed in K order through a
+                      workspace, and (with edge) edge tiles skip the MFMA blocks outside the matrix.  Stands
+                      in for what the reference gets from ranking tilings by rounds of blocks (num_wave,
+                      src/analyze.py:164-166).  Needs stages=3                                     */
 } rl_gemm_config;
+
+/* How a stream-K configuration splits one problem (rl_gemm_streamk_schedule). */
+typedef struct rl_streamk_schedule {
+  int grid;             /* workgroups launched */
+  int k_steps;          /* K steps per tile */
+  int tiles, tile_rows, tile_cols;
+  long units;           /* tiles * k_steps */
+  long cost;            /* sum over all units of their class cost; every workgroup gets cost / grid */
+  int class_tiles[4];   /* tiles per class: interior, right column, bottom row, corner */
+  int class_cost[4];    /* cost of one K step per class (MFMA blocks of the busiest wave, with a floor) */
+  size_t workspace_bytes, counter_bytes;
+} rl_streamk_schedule;
+
+/* One run of K steps of one tile, as a workgroup of a stream-K launch works it. */
+typedef struct rl_streamk_segment {
+  int tile_class, tile, tile_m, tile_n;
+  int k_begin, k_end;        /* K steps [k_begin, k_end) of the tile */
+  int pieces;                /* workgroups that share the tile (1: this segment is the whole tile) */
+  int first_workgroup;       /* the one with the tile's first K steps; the pieces follow in workgroup order */
+  int slot;                  /* workspace slot this piece is stored in, -1 if pieces == 1 */
+} rl_streamk_segment;
 
 /* ---- library / device ---------------------------------------------------------------------- */
 
@@ -173,6 +200,10 @@ int rl_gemm_plan_lds_bytes(const rl_gemm_plan* plan);
  * rl_gemm_plan_create fails with text when it is below rl_gemm_plan_lds_bytes. */
 int rl_gemm_plan_lds_limit(const rl_gemm_plan* plan);
 int rl_gemm_plan_threads(const rl_gemm_plan* plan);
+/* What hiprtc printed when it compiled the plan's kernel ("" if nothing, or if the code object came
+ * from the on-disk cache); owned by the library, valid while the plan is.  The counterpart of the IR
+ * dumps of src/roller.py:480-495. */
+const char* rl_gemm_plan_build_log(const rl_gemm_plan* plan);
 /* Kernel resource usage read from the code object's metadata (-1 if unknown). */
 int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int* sgprs,
                            int* spilled, int* scratch_bytes);
@@ -190,6 +221,30 @@ int rl_gemm_plans_clear(void);
  * K==0 writes zeros (or leaves C when accumulating). */
 int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
                         int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream);
+
+/* Stream-K plans (cfg.streamk > 0) need a workspace: arrival counters (one unsigned per tile, zero
+ * before a launch; the kernel leaves them at zero) followed by two slots of bm*bn floats per
+ * workgroup.  rl_gemm_plan_launch takes it from the library, which keeps one per stream (allocated or
+ * grown on first need, which synchronises that stream; launches on one stream run in order, and
+ * launches on different streams use different workspaces).  rl_gemm_plan_launch_ws takes it from the
+ * caller: `workspace` is device memory, 256-byte aligned, of at least rl_gemm_plan_workspace_bytes
+ * bytes, whose first *counter_bytes bytes were zero before its first use; launches that share a
+ * workspace must not overlap on the device.  For a plan without streamk both behave like
+ * rl_gemm_plan_launch and the workspace is ignored (bytes = 0).  No counterpart in the reference
+ * (src/roller.py:545-550 launches one block per tile). */
+int rl_gemm_plan_workspace_bytes(const rl_gemm_plan* plan, int M, int N, int K, size_t* bytes, size_t* counter_bytes);
+int rl_gemm_plan_launch_ws(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
+                           int M, int N, int K, int lda, int ldb, int ldc, void* workspace,
+                           size_t workspace_bytes, rl_stream stream);
+
+/* The split of an M x N x K problem under a stream-K configuration on a device with `compute_units`
+ * CUs, and the segments that workgroup `workgroup` works (at most `capacity` are written, *count
+ * receives how many there are).  Host arithmetic only (no device needed): what the policy's cost
+ * model and the tests read.  Replace the grid_size / num_wave fields of TileDict (src/analyze.py:150-166). */
+int rl_gemm_streamk_schedule(const rl_gemm_config* cfg, int M, int N, int K, int compute_units,
+                             rl_streamk_schedule* out);
+int rl_gemm_streamk_segments(const rl_gemm_config* cfg, int M, int N, int K, int compute_units,
+                             int workgroup, rl_streamk_segment* out, int capacity, int* count);
 
 /* One call for hosts that do not keep plans: plan_create (cached) + plan_launch. */
 int rl_gemm_f32(const rl_gemm_config* cfg, const float* A, const float* B, float* C, int M,

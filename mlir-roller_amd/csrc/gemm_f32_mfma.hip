@@ -47,6 +47,14 @@
 //               instead the 16-byte chunks of every A row are XOR-swizzled with the row number
 //               (on the load side by choosing which global chunk a lane fetches, on the read
 //               side in the fragment address), which keeps the 128-bit A reads conflict-free.
+//   STREAMK     0 = one workgroup per tile of C.  n > 0 = a fixed grid of n workgroups per CU, each of
+//               which works through an equal share of all (tile, K step) units, contiguous in K
+//               (gemm_sk_decode.inc).  A tile whose K range is split over workgroups is summed through
+//               a workspace: every piece is stored there, an arrival counter per tile tells the last
+//               piece in, and that workgroup adds the pieces in K order and writes C -- the same
+//               order whoever arrives last, so results are bit-identical from run to run.  With EDGE,
+//               tiles on the right and bottom edges skip the MFMA blocks that lie outside the matrix
+//               (their K steps then cost less, which the split accounts for).  Needs STAGES == 3.
 //   TRANS_B     1 = the second operand is given transposed, Bt[N][ldb >= K] (K contiguous, the
 //               layout in which the policy models both inputs, /root/reference/src/analyze.py:33-41).
 //               Its tile then sits in LDS like the A tile ([BN][BK+PAD_B], swizzled under DIRECT)
@@ -74,8 +82,8 @@
 // load issues beside the MFMAs for free, an instruction of the vector ALU (an address add, a
 // compare, a select) takes MFMA issue time, and the loop of the aligned 128-bit kernels has none.
 //
-// Summation order is fixed by (BK, MI) alone; there is no split-K and no atomics, so results are
-// bit-identical from run to run.
+// Summation order is fixed by (BK, MI) alone (with STREAMK: and by the split, a function of the
+// problem size and the grid), never by timing, so results are bit-identical from run to run.
 
 #ifndef __HIPCC_RTC__  // hiprtc pre-includes the device runtime declarations
 #include <hip/hip_runtime.h>
@@ -134,6 +142,9 @@
 #endif
 #ifndef TRANS_B
 #define TRANS_B 0
+#endif
+#ifndef STREAMK
+#define STREAMK 0
 #endif
 
 #define EDGE_K (EDGE == 1) /* the K extent may be ragged as well */
@@ -199,6 +210,7 @@ static_assert(NT <= 1024, "at most 16 waves per workgroup");
 static_assert(STAGES >= 1 && STAGES <= 5, "pipeline depth 1 to 5");
 static_assert(STAGES <= 3 || DIRECT, "more than two LDS buffers only with direct-to-LDS loads");
 static_assert(VEC == 4 || VEC == 1, "global access width");
+static_assert(STREAMK >= 0 && (!STREAMK || STAGES == 3), "the stream-K variant is built on the pipelined loop with two LDS buffers");
 static_assert(!DIRECT || (STAGES >= 3 && VEC == 4 && PAD_A == 0 && PAD_B == 0), "DIRECT needs STAGES>=3, VEC=4, no padding");
 /* Waiting for "all but the newest n tiles" counts this wave's outstanding loads, which is exact
  * only if every wave issues the same number of loads per tile. */
@@ -237,6 +249,12 @@ typedef v4f acc_t;
 #endif
 
 #define DEV static __device__ __forceinline__
+
+#if STREAMK
+#ifndef SK_DECODE_INCLUDED   /* the JIT path of the library puts the text in front of this file */
+#include "gemm_sk_decode.inc"
+#endif
+#endif
 
 // first block and width of B-read segment s
 DEV constexpr int seg_first(int s) { return s < NSEG4 ? 4 * s : (s == NSEG4 && HAS_SEG2 ? 4 * NSEG4 : TN - 1); }
@@ -385,7 +403,13 @@ DEV bool tile_of_workgroup(int nbm, int nbn, int& tile_m, int& tile_n) {
 
 extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const float* __restrict__ A, const float* __restrict__ B, float* __restrict__ C,
-    int M, int N, int K, int lda, int ldb, int ldc) {
+    int M, int N, int K, int lda, int ldb, int ldc
+#if STREAMK
+    // workspace: one slot of BM*BN floats per piece of a split tile (two per workgroup); one arrival
+    // counter per tile, zero before the launch and zero again when it ends; the split
+    , float* __restrict__ sk_slots, unsigned* __restrict__ sk_arrivals, const sk_params sk
+#endif
+) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
 
   const int tid = threadIdx.y * blockDim.x + threadIdx.x;
@@ -396,10 +420,47 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   const int lr = lane % MI;  // row of A / column slot of B inside an MFMA block
   const int lg = lane / MI;  // k group inside an MFMA
 
+#if STREAMK
+  // This workgroup's share of the (tile, K step) units, one segment (a run of K steps of one tile) at
+  // a time.  All of it is wave-uniform scalar arithmetic.
+  unsigned wg = blockIdx.x;
+  if (wg >= sk.grid) return;
+#if SWZ & 1
+  {
+    // workgroups are dealt to the XCDs round-robin: give every XCD one contiguous stretch of the units
+    const unsigned per = (sk.grid + NXCD - 1) / NXCD;
+    unsigned tall = sk.grid % NXCD;
+    if (tall == 0) tall = NXCD;
+    const unsigned xcd = wg % NXCD, loc = wg / NXCD;
+    wg = xcd < tall ? xcd * per + loc : tall * per + (xcd - tall) * (per - 1) + loc;
+  }
+#endif
+  unsigned sk_unit = sk_unit_at(sk, sk_virtual_start(sk, wg));
+  const unsigned sk_end = sk_unit_at(sk, sk_virtual_start(sk, wg + 1));
+  for (bool again = false; sk_unit < sk_end; again = true) {
+  const sk_segment seg = sk_segment_at(sk, sk_unit, sk_end);
+  sk_unit += seg.ke - seg.kb;
+  const int tile_m = (int)seg.tile_m, tile_n = (int)seg.tile_n;
+  const int kb = (int)seg.kb;                       // first K step of the segment
+  const bool skip_blocks = EDGE && seg.cls != 0;    // an edge tile that leaves out the MFMA blocks outside the matrix
+  if (again) __syncthreads();                       // every wave is done with the LDS tiles of the previous segment
+#else
   const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
   int tile_m, tile_n;
   if (!tile_of_workgroup(nbm, nbn, tile_m, tile_n)) return;
+  constexpr int kb = 0;
+  constexpr bool skip_blocks = false;
+  {
+#endif
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  // MFMA blocks of this wave that reach into the matrix (all of them unless blocks are skipped)
+  const int tm_act = !skip_blocks ? TM : (M - m0 - wm0 <= 0 ? 0 : (M - m0 - wm0 + MI - 1) / MI < TM ? (M - m0 - wm0 + MI - 1) / MI : TM);
+  // (a B read feeds the blocks of a segment column by column -- block e owns every w-th column -- so
+  // along N whole segments stay or go: tn_act is the end of the last segment that reaches into the matrix)
+  const int tn_need = N - n0 - wn0 <= 0 ? 0 : (N - n0 - wn0 + MI - 1) / MI;
+  const int tn_act = !skip_blocks ? TN
+                     : tn_need <= 4 * NSEG4 ? (tn_need + 3) / 4 * 4
+                     : (HAS_SEG2 && tn_need <= 4 * NSEG4 + 2) ? 4 * NSEG4 + 2 : TN;
 
   // ---- global -> register staging: per-thread loop-invariant offsets ----
   unsigned a_goff[A_PER_T], b_goff[B_PER_T];
@@ -449,23 +510,33 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
   }
 
-  const float* Ag = A + (long)m0 * lda;
-  long a_rem = ((long)(M - m0 - 1) * lda + K) * 4;        // valid bytes from Ag to the end of A
+  // The K loop below counts its steps from the segment's first one: operand bases start there and
+  // Kl is what is left of K from there on (all of K, from the start, unless STREAMK).
+  const int Kl = K - kb * BK;
 #if TRANS_B
-  const float* Bg = B + (long)n0 * ldb;
-  long b_rem = ((long)(N - n0 - 1) * ldb + K) * 4;        // valid bytes from Bg to the end of Bt
 #define B_STEP(k0) (long)(k0)                             /* floats from Bg to K step k0 */
 #else
-  const float* Bg = B + n0;
-  long b_rem = ((long)(K - 1) * ldb + (N - n0)) * 4;      // valid bytes from Bg to the end of B
 #define B_STEP(k0) ((long)(k0) * ldb)
+#endif
+  const float* Ag = A + (long)m0 * lda + kb * BK;
+  long a_rem = ((long)(M - m0 - 1) * lda + Kl) * 4;       // valid bytes from Ag to the end of A
+#if TRANS_B
+  const float* Bg = B + (long)n0 * ldb + B_STEP(kb * BK);
+  long b_rem = ((long)(N - n0 - 1) * ldb + Kl) * 4;       // valid bytes from Bg to the end of Bt
+#else
+  const float* Bg = B + n0 + B_STEP(kb * BK);
+  long b_rem = ((long)(Kl - 1) * ldb + (N - n0)) * 4;     // valid bytes from Bg to the end of B
 #endif
 
 #if !DIRECT
   v4f ra[A_PER_T], rb[B_PER_T];
 #endif
 
+#if STREAMK
+  const int KT = (int)(seg.ke - seg.kb);                  // K steps of this segment
+#else
   const int KT = (K + BK - 1) / BK;
+#endif
 
 #if DIRECT
   // Issues the loads of K step kt straight into LDS buffer `stage`.  Instruction i of a wave
@@ -485,7 +556,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < A_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (A_UNITS % NT == 0 || first < A_UNITS) {
-        const bool ok = a_ok[i] && (!KTEST || k0 + a_kcol[i] < K);
+        const bool ok = a_ok[i] && (!KTEST || k0 + a_kcol[i] < Kl);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr_t)(As + first * 4), 16, ok ? a_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -493,7 +564,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < B_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (B_UNITS % NT == 0 || first < B_UNITS) {
-        const bool ok = b_ok[i][0] && (!KTEST || k0 + b_krow[i] < K);  // K % 4 == 0: a chunk is in or out as a whole
+        const bool ok = b_ok[i][0] && (!KTEST || k0 + b_krow[i] < Kl);  // K % 4 == 0: a chunk is in or out as a whole
         __builtin_amdgcn_raw_ptr_buffer_load_lds(br, (lds_ptr_t)(Bs + first * 4), 16, ok ? b_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -514,21 +585,21 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int i = 0; i < A_PER_T; ++i) {
       const int k = k0 + a_kcol[i];
       ra[i] = load_unit<!KTEST>(ar, a_goff[i],
-                                a_ok[i] && (!KTEST || k + 0 < K), a_ok[i] && (!KTEST || k + 1 < K),
-                                a_ok[i] && (!KTEST || k + 2 < K), a_ok[i] && (!KTEST || k + 3 < K));
+                                a_ok[i] && (!KTEST || k + 0 < Kl), a_ok[i] && (!KTEST || k + 1 < Kl),
+                                a_ok[i] && (!KTEST || k + 2 < Kl), a_ok[i] && (!KTEST || k + 3 < Kl));
     }
 #pragma unroll
     for (int i = 0; i < B_PER_T; ++i) {
 #if TRANS_B
       const int k = k0 + b_krow[i];
       rb[i] = load_unit<!KTEST>(br, b_goff[i],
-                                b_ok[i][0] && (!KTEST || k + 0 < K), b_ok[i][1] && (!KTEST || k + 1 < K),
-                                b_ok[i][2] && (!KTEST || k + 2 < K), b_ok[i][3] && (!KTEST || k + 3 < K));
+                                b_ok[i][0] && (!KTEST || k + 0 < Kl), b_ok[i][1] && (!KTEST || k + 1 < Kl),
+                                b_ok[i][2] && (!KTEST || k + 2 < Kl), b_ok[i][3] && (!KTEST || k + 3 < Kl));
 #else
       // Columns at or beyond N only ever meet columns of C that are not stored, so a unit that
       // straddles N needs no zeroing: it is loaded if its first column is inside (what lies
       // past the end of the last row of B is beyond the range and comes back as zero).
-      const bool kin = !KTEST || k0 + b_krow[i] < K;
+      const bool kin = !KTEST || k0 + b_krow[i] < Kl;
       rb[i] = load_unit<true>(br, b_goff[i], b_ok[i][0] && kin, false, false, false);
 #endif
     }
@@ -611,13 +682,19 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     }
 #endif
   };
-  auto mfma_frags = [&](const frag_t& f, int t0 = 0, int t1 = 4) __attribute__((always_inline)) {
+  // SKIP (a compile-time 0/1): leave out the blocks at or beyond (tm_act, tn_act) -- a wave-uniform
+  // test per row and per block, which costs scalar branches and the static interleave, so only the
+  // edge tiles of the stream-K variant take this form.
+  auto mfma_frags = [&](auto skip, const frag_t& f, int t0 = 0, int t1 = 4) __attribute__((always_inline)) {
+    constexpr bool SKIP = decltype(skip)::value;
 #pragma unroll
     for (int t = t0; t < t1; ++t)
 #pragma unroll
-      for (int bi = 0; bi < TM; ++bi)
+      for (int bi = 0; bi < TM; ++bi) {
+        if (SKIP && bi >= tm_act) continue;
 #pragma unroll
         for (int bj = 0; bj < TN; ++bj) {
+          if (SKIP && bj >= tn_act) continue;
 #if TRANS_B
           const float bval = f.b[bj][t];
 #else
@@ -625,11 +702,13 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
           acc[bi][bj] = MFMA(f.a[bi][t], bval, acc[bi][bj]);
         }
+      }
   };
 
   // ---- main loop ----
 #if STAGES >= 3
-  if (KT > 0) {
+  auto main_loop = [&](auto skip) __attribute__((always_inline)) {
+    constexpr bool SKIP = decltype(skip)::value;
     // Software pipeline.  At the top of step kt: tile kt is in its LDS buffer, its first fragment
     // round is already in registers, and the staging registers hold tile kt+1 (loaded during step
     // kt-1).  Within the step each fragment round is read while the previous one is in the MFMA
@@ -678,31 +757,34 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
-        mfma_frags(fr[(P + r) & 1]);
+        mfma_frags(skip, fr[(P + r) & 1]);
       }
       // the last round is split around the barrier: its first half covers the LDS writes of
       // tile kt+1 and the global loads of tile kt+2, its second half the first reads of tile kt+1
       // (DIRECT: one quarter before the barrier, three after it, which leaves room to issue the
       // loads of tile kt+2 behind every second MFMA instead of every one: measured 0.3-0.8 % faster)
 #if DIRECT
-      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 1);
+      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 0, 1);
       // Tile kt+1 was requested LDS_BUFS-1 steps ago, straight into the next buffer; once every
       // wave's part has landed (the requests for later tiles may still be in flight) and all have
       // met, buffer `cur` is free again and takes tile kt+LDS_BUFS.
 #if SCHED
+      if constexpr (!SKIP) {
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
       // the barrier (and the wait for the LDS reads that comes with it) stays behind the MFMAs above:
       // left to float, it lands right behind the last read and the wave sits out that read's latency
       interleave_with_mfma<G / 4, 0, 0x100>();
       __builtin_amdgcn_sched_barrier(0);
+      }
 #endif
       WAIT_VMCNT((LDS_BUFS - 2) * LOADS_PER_TILE);
       __syncthreads();
       read_frags(fr[(P + SUPERS) & 1], nxt, 0);
       fetch_direct(ktail, kt + LDS_BUFS, cur);
-      mfma_frags(fr[(P + SUPERS - 1) & 1], 1, 4);
+      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 1, 4);
 #if SCHED
+      if constexpr (!SKIP) {
       {
         constexpr int REST = 3 * G / 4, PAIRED = R < REST ? R : REST, LEFT = REST - PAIRED;
         interleave_with_mfma<PAIRED, R, 0x100>();
@@ -712,22 +794,27 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
           interleave_with_mfma<LEFT, L, 0x020>();
         }
       }
+      }
 #endif
 #else
-      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
+      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 0, 2);
       stash(nxt);
       fetch(ktail, kt + 2);
 #if SCHED
+      if constexpr (!SKIP) {
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
       interleave_with_mfma<G / 4, W, 0x200>();
       interleave_with_mfma<G / 2 - G / 4, L, 0x020>();
+      }
 #endif
       __syncthreads();
       read_frags(fr[(P + SUPERS) & 1], nxt, 0);
-      mfma_frags(fr[(P + SUPERS - 1) & 1], 2, 4);
+      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 2, 4);
 #if SCHED
+      if constexpr (!SKIP) {
       interleave_with_mfma<G / 2, R, 0x100>();
+      }
 #endif
 #endif
     };
@@ -737,12 +824,14 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
-        mfma_frags(fr[(P + r) & 1]);
+        mfma_frags(skip, fr[(P + r) & 1]);
       }
-      mfma_frags(fr[(P + SUPERS - 1) & 1]);
+      mfma_frags(skip, fr[(P + SUPERS - 1) & 1]);
 #if SCHED
+      if constexpr (!SKIP) {
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
+      }
 #endif
 #if DIRECT
       WAIT_VMCNT(0);  // the (empty) requests for the tiles past the end have drained
@@ -775,6 +864,13 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (; kt + 1 < pipelined; kt += 2) pair(int_c<0>{}, kt);
 #endif
     last_step(int_c<0>{}, int_c<0>{}, pipelined);
+  };
+  if (KT > 0) {
+#if STREAMK && EDGE
+    if (skip_blocks) main_loop(int_c<1>{}); else main_loop(int_c<0>{});
+#else
+    main_loop(int_c<0>{});
+#endif
   }
 #else
   static_assert(!DIRECT, "DIRECT belongs to the pipelined loop");
@@ -783,7 +879,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int kk = 0; kk < BK; kk += KSUPER) {
       frag_t f;
       read_frags(f, stage, kk);
-      mfma_frags(f);
+      mfma_frags(int_c<0>{}, f);
     }
   };
   if (KT > 0) {
@@ -810,6 +906,65 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
 
   // ---- epilogue: every accumulator leaves once ----
+#if STREAMK
+  // A segment that covers its tile's whole K range stores C like the plain kernel.  Any other is a
+  // piece: it goes to this workgroup's slot in the workspace (slot 1 for a piece that starts the
+  // tile, which can only be the workgroup's last segment; slot 0 for one that starts inside the
+  // tile, which can only be its first), in the order the threads hold it.  The pieces of a tile
+  // belong to consecutive workgroups, first_wg .. first_wg + pieces - 1 in K order.  Whoever finds
+  // the tile's counter at pieces - 1 was last: it adds all pieces up in K order, its own included
+  // (read back, so the sum is formed the same way whoever comes last), stores C and clears the
+  // counter for the next launch.
+  bool store_c = true;
+  if (seg.kb != 0 || seg.ke != sk.kt) {
+    constexpr int CHUNKS = ACC_REGS / 4;            // 16-byte chunks per MFMA block and lane
+    const unsigned first_wg = sk_owner(sk, seg.first_unit);
+    const unsigned pieces = sk_owner(sk, seg.first_unit + sk.kt - 1) - first_wg + 1;
+    const unsigned my_slot = 2 * wg + (seg.kb == 0 ? 1 : 0);
+    {
+      const __amdgpu_buffer_rsrc_t wr = make_rsrc(sk_slots + (long)my_slot * (BM * BN), (long)BM * BN * 4);
+#pragma unroll
+      for (int bi = 0; bi < TM; ++bi)
+#pragma unroll
+        for (int bj = 0; bj < TN; ++bj)
+#pragma unroll
+          for (int c = 0; c < CHUNKS; ++c) {
+            const v4f v = {acc[bi][bj][4 * c], acc[bi][bj][4 * c + 1], acc[bi][bj][4 * c + 2], acc[bi][bj][4 * c + 3]};
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), wr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, 0);
+          }
+    }
+    // make the piece visible to the whole device, then count this workgroup in
+    __threadfence();
+    __syncthreads();
+    if (tid == 0)
+      lds[0] = __builtin_bit_cast(float, __hip_atomic_fetch_add(&sk_arrivals[seg.tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT));
+    __syncthreads();
+    const unsigned before = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(unsigned, lds[0]));
+    store_c = before == pieces - 1;
+    if (store_c) {
+      __threadfence();   // the other pieces, as their workgroups released them
+      auto add_piece = [&](auto is_first, unsigned slot) __attribute__((always_inline)) {
+        const __amdgpu_buffer_rsrc_t rr = make_rsrc(sk_slots + (long)slot * (BM * BN), (long)BM * BN * 4);
+#pragma unroll
+        for (int bi = 0; bi < TM; ++bi)
+#pragma unroll
+          for (int bj = 0; bj < TN; ++bj)
+#pragma unroll
+            for (int c = 0; c < CHUNKS; ++c) {
+              const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, 0));
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[bi][bj][4 * c + e] = decltype(is_first)::value ? v[e] : acc[bi][bj][4 * c + e] + v[e];
+            }
+      };
+      add_piece(int_c<1>{}, 2 * first_wg + 1);
+      for (unsigned piece = 1; piece < pieces; ++piece) add_piece(int_c<0>{}, 2 * (first_wg + piece));
+      if (tid == 0) __hip_atomic_store(&sk_arrivals[seg.tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  if (store_c) {
+#else
+  {
+#endif
   float* Cg = C + (long)m0 * ldc + n0;
   const __amdgpu_buffer_rsrc_t cr = make_rsrc(Cg, ((long)(M - m0 - 1) * ldc + (N - n0)) * 4);
 #pragma unroll
@@ -853,4 +1008,6 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
         }
       }
     }
+  }   // store_c
+  }   // segment
 }

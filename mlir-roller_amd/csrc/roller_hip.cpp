@@ -26,19 +26,28 @@
 #include <string>
 #include <vector>
 
-#ifndef RL_TEMPLATE_PATH
-#error "build with -DRL_TEMPLATE_PATH=\"<path to gemm_f32_mfma.hip>\""
+#if !defined(RL_TEMPLATE_PATH) || !defined(RL_SK_DECODE_PATH)
+#error "build with -DRL_TEMPLATE_PATH=\"<path to gemm_f32_mfma.hip>\" -DRL_SK_DECODE_PATH=\"<path to gemm_sk_decode.inc>\""
 #endif
 
-// The kernel template, byte for byte, NUL-terminated.
+// The kernel template and the work decomposition it includes, byte for byte, NUL-terminated.  The
+// decomposition is also compiled into this file: the host fills the launch parameters with the
+// same arithmetic that the workgroups decode them with.
 __asm__(
     ".section .rodata\n"
     ".global rl_gemm_template_begin\n"
     "rl_gemm_template_begin:\n"
     ".incbin \"" RL_TEMPLATE_PATH "\"\n"
     ".byte 0\n"
+    ".global rl_gemm_sk_decode_begin\n"
+    "rl_gemm_sk_decode_begin:\n"
+    ".incbin \"" RL_SK_DECODE_PATH "\"\n"
+    ".byte 0\n"
     ".previous\n");
 extern "C" const char rl_gemm_template_begin[];
+extern "C" const char rl_gemm_sk_decode_begin[];
+
+#include "gemm_sk_decode.inc"
 
 namespace {
 
@@ -71,6 +80,7 @@ std::shared_mutex g_plans_rw;
 std::atomic<bool> g_ready{false};  // read without the lock on every entry point
 std::atomic<int> g_device{-1};
 std::atomic<int> g_lds_limit{0};   // largest LDS allocation of one workgroup, read from the device at rl_init
+std::atomic<int> g_compute_units{0};
 std::string g_cache_dir;
 
 struct Plan {
@@ -81,6 +91,7 @@ struct Plan {
   int lds_limit = 0;  // dynamic LDS the runtime grants this function, read back after load
   int threads = 0;
   int vgprs = -1, agprs = -1, sgprs = -1, spilled = -1, scratch = -1;
+  std::string build_log;   // what hiprtc printed for this kernel ("" when the code object came from the disk cache)
 };
 
 }  // namespace
@@ -94,6 +105,13 @@ std::map<std::string, rl_gemm_plan*> g_plans;
 // stay allocated so that a handle a caller still holds is refused instead of dereferencing
 // freed memory.
 std::vector<rl_gemm_plan*> g_released_plans;
+
+// What hiprtc compiles: the work decomposition (which defines the guard that makes the template skip
+// its own #include of it) followed by the template.
+const std::string& jit_source() {
+  static const std::string text = std::string(rl_gemm_sk_decode_begin) + "\n" + rl_gemm_template_begin;
+  return text;
+}
 
 uint64_t fnv1a(const void* data, size_t n, uint64_t h) {
   const unsigned char* p = (const unsigned char*)data;
@@ -137,6 +155,8 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
       return fail(RL_ERR_INVALID_ARG, "direct=1 needs bm*bk and bk*bn to be multiples of 256 (whole waves of 16-byte units)");
   }
   if ((c.trans_b | 1) != 1) return fail(RL_ERR_INVALID_ARG, "trans_b is 0 or 1");
+  if (c.streamk < 0 || c.streamk > 8) return fail(RL_ERR_INVALID_ARG, "streamk is 0 (one workgroup per tile) or 1 to 8 workgroups per CU, got %d", c.streamk);
+  if (c.streamk && c.stages != 3) return fail(RL_ERR_INVALID_ARG, "streamk needs stages=3 (the pipelined loop with two LDS buffers), got stages=%d", c.stages);
   const int nt = 64 * (c.bm / c.wm) * (c.bn / c.wn);
   if (nt > 1024) return fail(RL_ERR_INVALID_ARG, "%d threads per workgroup exceed 1024", nt);
   const int bufs = c.stages >= 3 ? c.stages - 1 : c.stages;  // LDS buffers: 1, 2, 2, 3, 4
@@ -163,6 +183,7 @@ std::vector<std::string> config_options(const rl_gemm_config& c) {
   def("EDGE", c.edge); def("SWZ", c.swz); def("GROUP", c.group > 0 ? c.group : 1); def("ACCUM", c.accum);
   def("DIRECT", c.direct);
   def("TRANS_B", c.trans_b);
+  def("STREAMK", c.streamk);
   return o;
 }
 
@@ -172,12 +193,14 @@ std::string config_key(const rl_gemm_config& c) {
   return k;
 }
 
+const char* const kFixedOptions[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
+                                     "-Xclang", "-packed-fp32-ops"};
+
 int compile(const char* source, const char* name, const std::vector<std::string>& user_opts,
             std::vector<char>* code, std::string* log) {
   // Fixed part of the command line: the one target this library serves, and no packed-fp32
   // instruction selection.
-  std::vector<std::string> all = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature",
-                                  "-Xclang", "-packed-fp32-ops"};
+  std::vector<std::string> all(std::begin(kFixedOptions), std::end(kFixedOptions));
   all.insert(all.end(), user_opts.begin(), user_opts.end());
   std::vector<const char*> argv;
   for (const std::string& s : all) argv.push_back(s.c_str());
@@ -210,13 +233,20 @@ int compile(const char* source, const char* name, const std::vector<std::string>
 
 std::string cache_path(const rl_gemm_config& c) {
   if (g_cache_dir.empty()) return "";
-  int major = 0, minor = 0;
+  // everything that decides the code object: source text, template parameters, the fixed part of the
+  // command line, and the compiler -- hiprtc's own version and that of the HIP runtime it ships with
+  // (which carries the patch level and changes with every ROCm release)
+  int major = 0, minor = 0, runtime = 0;
   hiprtcVersion(&major, &minor);
-  const std::string key = config_key(c) + "|hiprtc " + std::to_string(major) + "." + std::to_string(minor);
-  uint64_t h1 = fnv1a(rl_gemm_template_begin, strlen(rl_gemm_template_begin), 14695981039346656037ull);
+  (void)hipRuntimeGetVersion(&runtime);
+  std::string key = config_key(c) + "|";
+  for (const char* o : kFixedOptions) key += std::string(o) + " ";
+  key += "|hiprtc " + std::to_string(major) + "." + std::to_string(minor) + " hip " + std::to_string(runtime);
+  const std::string& source = jit_source();
+  uint64_t h1 = fnv1a(source.data(), source.size(), 14695981039346656037ull);
   h1 = fnv1a(key.data(), key.size(), h1);
   uint64_t h2 = fnv1a(key.data(), key.size(), 0x9e3779b97f4a7c15ull);
-  h2 = fnv1a(rl_gemm_template_begin, strlen(rl_gemm_template_begin), h2);
+  h2 = fnv1a(source.data(), source.size(), h2);
   char name[64];
   snprintf(name, sizeof name, "gemm_%016llx%016llx.hsaco", (unsigned long long)h1, (unsigned long long)h2);
   return g_cache_dir + "/" + name;
@@ -277,7 +307,7 @@ bool strip_trailer(std::vector<char>* data) {
 // Code object for cfg: from the disk cache if present (unless use_cache is false), otherwise
 // compiled (and then cached).  *from_cache tells the caller which of the two it got.
 int code_for(const rl_gemm_config& c, std::vector<char>* code, float* compile_ms, bool use_cache = true,
-             bool* from_cache = nullptr) {
+             bool* from_cache = nullptr, std::string* build_log = nullptr) {
   if (compile_ms) *compile_ms = 0.0f;
   if (from_cache) *from_cache = false;
   const std::string path = cache_path(c);
@@ -288,7 +318,8 @@ int code_for(const rl_gemm_config& c, std::vector<char>* code, float* compile_ms
   code->clear();
   std::string log;
   const auto t0 = std::chrono::steady_clock::now();
-  int rc = compile(rl_gemm_template_begin, "gemm_f32_mfma.hip", config_options(c), code, &log);
+  int rc = compile(jit_source().c_str(), "gemm_f32_mfma.hip", config_options(c), code, &log);
+  if (build_log) *build_log = log;
   if (rc != RL_OK) return rc;
   if (compile_ms)
     *compile_ms = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -369,6 +400,208 @@ int opt_in_lds(hipFunction_t f, int bytes, int* granted) {
   return RL_OK;
 }
 
+
+// ---- stream-K: launch parameters and workspace -------------------------------------------------------
+
+sk_div make_div(unsigned d) {
+  // Division of any 32-bit x by the constant d >= 1 (Granlund & Montgomery, the form without a branch):
+  // l = ceil(log2 d), mul = floor(2^32 * (2^l - d) / d) + 1, x / d = (t + ((x - t) >> 1)) >> (l - 1) with
+  // t = mulhi(x, mul); d = 1 is the same formula with mul = 0 and both shifts 0.
+  sk_div out{0u, 0u};
+  if (d <= 1) return out;
+  unsigned l = 0;
+  while ((1ull << l) < d) ++l;
+  out.mul = (unsigned)((((1ull << l) - d) << 32) / d + 1);
+  out.sh = (1u << 8) | (l - 1);
+  return out;
+}
+
+// Cost of one K step of an edge tile relative to the MFMA blocks it keeps: below a quarter of a full
+// tile's blocks a step is bounded by its loads and barrier, not by its MFMAs.  Overridable for
+// experiments (percent of a full tile's cost).
+unsigned min_step_cost(unsigned full) {
+  static const int percent = [] {
+    const char* e = getenv("ROLLER_SK_MIN_COST_PERCENT");
+    const int v = e ? atoi(e) : 25;
+    return v < 1 ? 1 : (v > 100 ? 100 : v);
+  }();
+  const unsigned m = (full * (unsigned)percent + 99) / 100;
+  return m < 1 ? 1 : m;
+}
+
+// Fills *p for cfg on an M x N x K problem with `compute_units` CUs.  Edge classes exist when the
+// kernel predicates edges (cfg.edge) and the busiest wave of such a tile keeps fewer MFMA blocks than
+// a full tile has.  The grid is cfg.streamk workgroups per CU, cut down where the problem is too
+// small to give every workgroup one full-cost K step (the decoding relies on no share being empty).
+int sk_make_params(const rl_gemm_config& c, int M, int N, int K, int compute_units, sk_params* p, unsigned* tiles) {
+  if (!c.streamk) return fail(RL_ERR_INVALID_ARG, "not a stream-K configuration");
+  if (M <= 0 || N <= 0 || K <= 0) return fail(RL_ERR_INVALID_ARG, "stream-K needs M, N, K > 0 (M=%d N=%d K=%d)", M, N, K);
+  if (compute_units <= 0) return fail(RL_ERR_INVALID_ARG, "compute_units must be positive");
+  const unsigned long nbm = ((unsigned long)M + c.bm - 1) / c.bm, nbn = ((unsigned long)N + c.bn - 1) / c.bn;
+  const unsigned long kt = ((unsigned long)K + c.bk - 1) / c.bk;
+  const unsigned tm = c.wm / c.mi, tn = c.wn / c.mi, full = tm * tn;
+  const unsigned mrem = (unsigned)(M - (long)(nbm - 1) * c.bm), nrem = (unsigned)(N - (long)(nbn - 1) * c.bn);
+  // MFMA blocks that the wave at the tile's origin (the busiest one) keeps: block rows one by one, block
+  // columns by whole read segments (four blocks, then two, then one), as the kernel skips them
+  auto block_rows = [&](unsigned valid) {
+    const unsigned b = (valid + c.mi - 1) / c.mi;
+    return b < tm ? b : tm;
+  };
+  auto block_cols = [&](unsigned valid) {
+    const unsigned b = (valid + c.mi - 1) / c.mi, fours = tn / 4 * 4;
+    if (b <= fours) return (b + 3) / 4 * 4;
+    if ((tn % 4) / 2 && b <= fours + 2) return fours + 2;
+    return tn;
+  };
+  const unsigned floor_cost = min_step_cost(full);
+  auto cost = [&](unsigned rows, unsigned cols) {
+    const unsigned b = block_rows(rows) * block_cols(cols);
+    return b < floor_cost ? floor_cost : b;
+  };
+  const unsigned w_right = cost(c.bm, nrem), w_bottom = cost(mrem, c.bn), w_corner = cost(mrem, nrem);
+  const bool has_r = c.edge && nrem < (unsigned)c.bn && w_right < full;
+  const bool has_b = c.edge && mrem < (unsigned)c.bm && w_bottom < full;
+  const unsigned long nim = nbm - (has_b ? 1 : 0), nin = nbn - (has_r ? 1 : 0);
+  const unsigned long count[4] = {nim * nin, has_r ? nim : 0, has_b ? nin : 0, (has_r && has_b) ? 1ul : 0ul};
+  // a corner next to only one skipped edge belongs to that edge's class
+  const unsigned w[4] = {full, w_right, w_bottom, w_corner};
+  unsigned long u = 0, v = 0, t = 0, ub[5], vb[5], tb[4];
+  for (int k = 0; k < 4; ++k) {
+    ub[k] = u; vb[k] = v; tb[k] = t;
+    u += count[k] * kt; v += count[k] * kt * w[k]; t += count[k];
+  }
+  ub[4] = u; vb[4] = v;
+  if (v >= 0x7fffffffUL || u >= 0x7fffffffUL || nbm > 0xffffffUL || nbn > 0xffffffUL)
+    return fail(RL_ERR_INVALID_ARG, "problem too large for the 32-bit arithmetic of the stream-K split (%lu units of cost %lu)", u, v);
+  unsigned long grid = (unsigned long)compute_units * c.streamk;
+  if (grid > v / full) grid = v / full;     // every share at least one full-cost K step: no share is empty
+  if (grid < 1) grid = 1;
+  memset(p, 0, sizeof *p);
+  p->grid = (unsigned)grid; p->q = (unsigned)(v / grid); p->r = (unsigned)(v % grid); p->kt = (unsigned)kt;
+  p->nbm = (unsigned)nbm; p->nbn = (unsigned)nbn; p->nim = (unsigned)nim; p->nin = (unsigned)nin;
+  p->group = (c.swz & 2) ? (unsigned)(c.group > 0 ? c.group : 1) : 1u;
+  p->rows_last = (unsigned)(nim % p->group);
+  p->w0 = w[0]; p->w1 = w[1]; p->w2 = w[2]; p->w3 = w[3];
+  p->u1 = (unsigned)ub[1]; p->u2 = (unsigned)ub[2]; p->u3 = (unsigned)ub[3]; p->u4 = (unsigned)ub[4];
+  p->v1 = (unsigned)vb[1]; p->v2 = (unsigned)vb[2]; p->v3 = (unsigned)vb[3];
+  p->t1 = (unsigned)tb[1]; p->t2 = (unsigned)tb[2]; p->t3 = (unsigned)tb[3];
+  p->d_kt = make_div(p->kt); p->d_q = make_div(p->q); p->d_q1 = make_div(p->q + 1);
+  p->d_width = make_div(p->group * (p->nin ? p->nin : 1)); p->d_group = make_div(p->group);
+  p->d_rows_last = make_div(p->rows_last ? p->rows_last : 1);
+  p->d_w0 = make_div(w[0]); p->d_w1 = make_div(w[1]); p->d_w2 = make_div(w[2]); p->d_w3 = make_div(w[3]);
+  if (tiles) *tiles = (unsigned)t;
+  return RL_OK;
+}
+
+// Workspace of one stream-K launch: the arrival counters (one per tile, rounded up to 256 bytes),
+// then two slots of bm*bn floats per workgroup.
+size_t sk_counter_bytes(unsigned tiles) { return ((size_t)tiles * 4 + 255) / 256 * 256; }
+size_t sk_workspace_bytes(const rl_gemm_config& c, const sk_params& p, unsigned tiles) {
+  return sk_counter_bytes(tiles) + (size_t)2 * p.grid * c.bm * c.bn * 4;
+}
+
+// Workspaces the library owns, one per stream (launches on one stream run in order; launches on
+// different streams may overlap and must not share counters or slots).  Grown on demand, zeroed
+// when allocated (the kernels leave the counters at zero), freed never: a stream's last workspace
+// lives until the process ends.
+struct Workspace {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+};
+std::map<hipStream_t, Workspace> g_workspaces;
+std::mutex g_workspaces_mutex;   // (its own lock: launches hold the plan table's shared lock when they get here)
+
+int workspace_for(hipStream_t stream, size_t bytes, void** out) {
+  std::lock_guard<std::mutex> lock(g_workspaces_mutex);
+  Workspace& w = g_workspaces[stream];
+  if (w.bytes < bytes) {
+    if (w.ptr) {
+      // the old one may still be in use by a launch queued on this stream
+      HIP_TRY(hipStreamSynchronize(stream));
+      HIP_TRY(hipFree(w.ptr));
+      w = Workspace();
+    }
+    const size_t want = bytes + bytes / 4;   // head room, so that a slightly larger problem does not reallocate
+    HIP_TRY(hipMalloc(&w.ptr, want));
+    HIP_TRY(hipMemset(w.ptr, 0, want));
+    w.bytes = want;
+  }
+  *out = w.ptr;
+  return RL_OK;
+}
+
+enum WorkspaceKind { WS_LIBRARY, WS_CALLER };
+
+// Argument checks and launch shared by the plan entry points.  A stream-K plan takes its workspace
+// from the library (one per stream) or from the caller.
+int launch_plan(const rl_gemm_plan* plan, const float* A, const float* B, float* C, int M, int N, int K,
+                int lda, int ldb, int ldc, rl_stream stream, WorkspaceKind kind, void* user_ws, size_t user_ws_bytes) {
+  if (!plan) return fail(RL_ERR_INVALID_ARG, "plan is NULL");
+  READY_OR_RETURN();
+  std::shared_lock<std::shared_mutex> in_flight(g_plans_rw);
+  if (!plan->func) return fail(RL_ERR_INVALID_ARG, "plan was released by rl_gemm_plans_clear");
+  const rl_gemm_config& c = plan->cfg;
+  if (M < 0 || N < 0 || K < 0) return fail(RL_ERR_INVALID_ARG, "negative dimension (M=%d N=%d K=%d)", M, N, K);
+  if (M == 0 || N == 0) return RL_OK;
+  if (!C || (K > 0 && (!A || !B))) return fail(RL_ERR_INVALID_ARG, "NULL matrix pointer");
+  if (lda < K || ldb < (c.trans_b ? K : N) || ldc < N)
+    return fail(RL_ERR_INVALID_ARG, "leading dimension too small (lda=%d K=%d, ldb=%d ldc=%d N=%d, trans_b=%d)", lda, K, ldb, ldc, N, c.trans_b);
+  if (c.vec == 4) {
+    if (K % 4 || N % 4 || lda % 4 || ldb % 4 || ldc % 4)
+      return fail(RL_ERR_INVALID_ARG, "vec=4 kernel needs K, N, lda, ldb, ldc to be multiples of 4 (K=%d N=%d lda=%d ldb=%d ldc=%d)", K, N, lda, ldb, ldc);
+    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15)
+      return fail(RL_ERR_INVALID_ARG, "vec=4 kernel needs 16-byte aligned A, B and C");
+  } else if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 3) {
+    return fail(RL_ERR_INVALID_ARG, "A, B and C must be 4-byte aligned");
+  }
+  if (!c.edge && (M % c.bm || N % c.bn || K % c.bk))
+    return fail(RL_ERR_INVALID_ARG, "edge=0 kernel needs bm|M, bn|N, bk|K (tile %dx%dx%d, problem %dx%dx%d)", c.bm, c.bn, c.bk, M, N, K);
+  if (c.edge == 2 && K % c.bk)
+    return fail(RL_ERR_INVALID_ARG, "edge=2 kernel needs bk|K (bk=%d, K=%d)", c.bk, K);
+  // In-tile byte offsets are 32-bit inside the kernel; 0x80000000 is reserved as "out of range".
+  const long lim = 0x7fffffffL;
+  if ((long)c.bm * lda * 4 + (long)c.bk * 4 > lim || (c.trans_b ? (long)c.bn * ldb * 4 + (long)c.bk * 4 : (long)c.bk * ldb * 4 + (long)c.bn * 4) > lim ||
+      (long)c.bm * ldc * 4 + (long)c.bn * 4 > lim)
+    return fail(RL_ERR_INVALID_ARG, "leading dimension too large for 32-bit in-tile offsets");
+  const long nbm = ((long)M + c.bm - 1) / c.bm, nbn = ((long)N + c.bn - 1) / c.bn;
+  if (nbn > 0x7fffffffL || nbm > 65535 || nbm * nbn > lim)
+    return fail(RL_ERR_INVALID_ARG, "tile grid %ldx%ld too large", nbn, nbm);
+
+  if (!c.streamk) {
+    void* args[] = {(void*)&A, (void*)&B, (void*)&C, &M, &N, &K, &lda, &ldb, &ldc};
+    HIP_TRY(hipModuleLaunchKernel(plan->func, (unsigned)nbn, (unsigned)nbm, 1, (unsigned)plan->threads, 1, 1,
+                                  (unsigned)plan->lds_bytes, (hipStream_t)stream, args, nullptr));
+    return RL_OK;
+  }
+
+  if (K == 0) {
+    // no K step to hand out: C = 0 (or C unchanged when accumulating), without the kernel
+    if (!c.accum) HIP_TRY(hipMemset2DAsync(C, (size_t)ldc * 4, 0, (size_t)N * 4, (size_t)M, (hipStream_t)stream));
+    return RL_OK;
+  }
+  sk_params sp;
+  unsigned tiles = 0;
+  int rc = sk_make_params(c, M, N, K, g_compute_units.load(), &sp, &tiles);
+  if (rc) return rc;
+  const size_t need = sk_workspace_bytes(c, sp, tiles);
+  void* ws = nullptr;
+  if (kind == WS_CALLER) {
+    if (!user_ws || user_ws_bytes < need)
+      return fail(RL_ERR_INVALID_ARG, "stream-K launch needs a workspace of %zu bytes (rl_gemm_plan_workspace_bytes), got %zu", need, user_ws ? user_ws_bytes : (size_t)0);
+    if ((uintptr_t)user_ws & 255) return fail(RL_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
+    ws = user_ws;
+  } else {
+    rc = workspace_for((hipStream_t)stream, need, &ws);
+    if (rc) return rc;
+  }
+  unsigned* arrivals = (unsigned*)ws;
+  float* slots = (float*)((char*)ws + sk_counter_bytes(tiles));
+  void* args[] = {(void*)&A, (void*)&B, (void*)&C, &M, &N, &K, &lda, &ldb, &ldc, &slots, &arrivals, &sp};
+  HIP_TRY(hipModuleLaunchKernel(plan->func, sp.grid, 1, 1, (unsigned)plan->threads, 1, 1,
+                                (unsigned)plan->lds_bytes, (hipStream_t)stream, args, nullptr));
+  return RL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -395,6 +628,7 @@ int rl_init(int device) {
   if (hipDeviceGetAttribute(&attr, hipDeviceAttributeMaxSharedMemoryPerBlock, device) == hipSuccess && attr > lds_limit)
     lds_limit = attr;
   g_lds_limit = lds_limit;
+  g_compute_units = prop.multiProcessorCount;
   g_device = device;
   g_ready = true;
   return RL_OK;
@@ -602,7 +836,7 @@ int rl_sync(void) {
   return RL_OK;
 }
 
-const char* rl_gemm_template_source(void) { return rl_gemm_template_begin; }
+const char* rl_gemm_template_source(void) { return jit_source().c_str(); }
 
 int rl_gemm_config_check(const rl_gemm_config* cfg, int* lds_bytes, int* threads) {
   if (!cfg) return fail(RL_ERR_INVALID_ARG, "cfg is NULL");
@@ -660,10 +894,12 @@ int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* co
   }
   std::vector<char> code;
   bool from_cache = false;
-  rc = code_for(*cfg, &code, compile_ms, true, &from_cache);
+  std::string build_log;
+  rc = code_for(*cfg, &code, compile_ms, true, &from_cache, &build_log);
   if (rc) return rc;
 
   rl_gemm_plan* p = new rl_gemm_plan();
+  p->build_log = build_log;
   p->cfg = *cfg;
   p->lds_bytes = lds;
   p->threads = threads;
@@ -678,7 +914,7 @@ int rl_gemm_plan_create(const rl_gemm_config* cfg, rl_gemm_plan** out, float* co
     p->module = nullptr;
     p->func = nullptr;
     from_cache = false;
-    rc = code_for(*cfg, &code, compile_ms, false, nullptr);
+    rc = code_for(*cfg, &code, compile_ms, false, nullptr, &p->build_log);
     if (rc) {
       delete p;
       return rc;
@@ -731,6 +967,8 @@ int rl_gemm_plan_resources(const rl_gemm_plan* plan, int* vgprs, int* agprs, int
   return RL_OK;
 }
 
+const char* rl_gemm_plan_build_log(const rl_gemm_plan* plan) { return plan ? plan->build_log.c_str() : ""; }
+
 int rl_gemm_plans_clear(void) {
   READY_OR_RETURN();
   std::lock_guard<std::mutex> lock(g_mutex);
@@ -753,40 +991,89 @@ int rl_gemm_plans_clear(void) {
 
 int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
                         int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream) {
-  if (!plan) return fail(RL_ERR_INVALID_ARG, "plan is NULL");
-  READY_OR_RETURN();
-  std::shared_lock<std::shared_mutex> in_flight(g_plans_rw);
-  if (!plan->func) return fail(RL_ERR_INVALID_ARG, "plan was released by rl_gemm_plans_clear");
-  const rl_gemm_config& c = plan->cfg;
-  if (M < 0 || N < 0 || K < 0) return fail(RL_ERR_INVALID_ARG, "negative dimension (M=%d N=%d K=%d)", M, N, K);
-  if (M == 0 || N == 0) return RL_OK;
-  if (!C || (K > 0 && (!A || !B))) return fail(RL_ERR_INVALID_ARG, "NULL matrix pointer");
-  if (lda < K || ldb < (c.trans_b ? K : N) || ldc < N)
-    return fail(RL_ERR_INVALID_ARG, "leading dimension too small (lda=%d K=%d, ldb=%d ldc=%d N=%d, trans_b=%d)", lda, K, ldb, ldc, N, c.trans_b);
-  if (c.vec == 4) {
-    if (K % 4 || N % 4 || lda % 4 || ldb % 4 || ldc % 4)
-      return fail(RL_ERR_INVALID_ARG, "vec=4 kernel needs K, N, lda, ldb, ldc to be multiples of 4 (K=%d N=%d lda=%d ldb=%d ldc=%d)", K, N, lda, ldb, ldc);
-    if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15)
-      return fail(RL_ERR_INVALID_ARG, "vec=4 kernel needs 16-byte aligned A, B and C");
-  } else if (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 3) {
-    return fail(RL_ERR_INVALID_ARG, "A, B and C must be 4-byte aligned");
-  }
-  if (!c.edge && (M % c.bm || N % c.bn || K % c.bk))
-    return fail(RL_ERR_INVALID_ARG, "edge=0 kernel needs bm|M, bn|N, bk|K (tile %dx%dx%d, problem %dx%dx%d)", c.bm, c.bn, c.bk, M, N, K);
-  if (c.edge == 2 && K % c.bk)
-    return fail(RL_ERR_INVALID_ARG, "edge=2 kernel needs bk|K (bk=%d, K=%d)", c.bk, K);
-  // In-tile byte offsets are 32-bit inside the kernel; 0x80000000 is reserved as "out of range".
-  const long lim = 0x7fffffffL;
-  if ((long)c.bm * lda * 4 + (long)c.bk * 4 > lim || (c.trans_b ? (long)c.bn * ldb * 4 + (long)c.bk * 4 : (long)c.bk * ldb * 4 + (long)c.bn * 4) > lim ||
-      (long)c.bm * ldc * 4 + (long)c.bn * 4 > lim)
-    return fail(RL_ERR_INVALID_ARG, "leading dimension too large for 32-bit in-tile offsets");
-  const long nbm = ((long)M + c.bm - 1) / c.bm, nbn = ((long)N + c.bn - 1) / c.bn;
-  if (nbn > 0x7fffffffL || nbm > 65535 || nbm * nbn > lim)
-    return fail(RL_ERR_INVALID_ARG, "tile grid %ldx%ld too large", nbn, nbm);
+  return launch_plan(plan, A, B, C, M, N, K, lda, ldb, ldc, stream, WS_LIBRARY, nullptr, 0);
+}
 
-  void* args[] = {(void*)&A, (void*)&B, (void*)&C, &M, &N, &K, &lda, &ldb, &ldc};
-  HIP_TRY(hipModuleLaunchKernel(plan->func, (unsigned)nbn, (unsigned)nbm, 1, (unsigned)plan->threads, 1, 1,
-                                (unsigned)plan->lds_bytes, (hipStream_t)stream, args, nullptr));
+int rl_gemm_plan_launch_ws(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
+                           int M, int N, int K, int lda, int ldb, int ldc, void* workspace,
+                           size_t workspace_bytes, rl_stream stream) {
+  return launch_plan(plan, A, B, C, M, N, K, lda, ldb, ldc, stream, WS_CALLER, workspace, workspace_bytes);
+}
+
+int rl_gemm_plan_workspace_bytes(const rl_gemm_plan* plan, int M, int N, int K, size_t* bytes, size_t* counter_bytes) {
+  if (!plan || !bytes) return fail(RL_ERR_INVALID_ARG, "rl_gemm_plan_workspace_bytes: NULL argument");
+  *bytes = 0;
+  if (counter_bytes) *counter_bytes = 0;
+  if (!plan->cfg.streamk || M <= 0 || N <= 0 || K <= 0) return RL_OK;
+  READY_OR_RETURN();
+  sk_params sp;
+  unsigned tiles = 0;
+  int rc = sk_make_params(plan->cfg, M, N, K, g_compute_units.load(), &sp, &tiles);
+  if (rc) return rc;
+  *bytes = sk_workspace_bytes(plan->cfg, sp, tiles);
+  if (counter_bytes) *counter_bytes = sk_counter_bytes(tiles);
+  return RL_OK;
+}
+
+int rl_gemm_streamk_schedule(const rl_gemm_config* cfg, int M, int N, int K, int compute_units,
+                             rl_streamk_schedule* out) {
+  if (!cfg || !out) return fail(RL_ERR_INVALID_ARG, "rl_gemm_streamk_schedule: NULL argument");
+  int rc = check_config(*cfg, nullptr, nullptr);
+  if (rc) return rc;
+  sk_params sp;
+  unsigned tiles = 0;
+  rc = sk_make_params(*cfg, M, N, K, compute_units, &sp, &tiles);
+  if (rc) return rc;
+  memset(out, 0, sizeof *out);
+  out->grid = (int)sp.grid;
+  out->k_steps = (int)sp.kt;
+  out->tiles = (int)tiles;
+  out->tile_rows = (int)sp.nbm;
+  out->tile_cols = (int)sp.nbn;
+  out->units = (long)sp.u4;
+  out->cost = (long)sp.grid * sp.q + sp.r;
+  const unsigned first[5] = {0u, sp.u1, sp.u2, sp.u3, sp.u4}, w[4] = {sp.w0, sp.w1, sp.w2, sp.w3};
+  for (int k = 0; k < 4; ++k) {
+    out->class_tiles[k] = (int)((first[k + 1] - first[k]) / sp.kt);
+    out->class_cost[k] = (int)w[k];
+  }
+  out->workspace_bytes = sk_workspace_bytes(*cfg, sp, tiles);
+  out->counter_bytes = sk_counter_bytes(tiles);
+  return RL_OK;
+}
+
+int rl_gemm_streamk_segments(const rl_gemm_config* cfg, int M, int N, int K, int compute_units,
+                             int workgroup, rl_streamk_segment* out, int capacity, int* count) {
+  if (!cfg || !count || (capacity > 0 && !out)) return fail(RL_ERR_INVALID_ARG, "rl_gemm_streamk_segments: NULL argument");
+  int rc = check_config(*cfg, nullptr, nullptr);
+  if (rc) return rc;
+  sk_params sp;
+  rc = sk_make_params(*cfg, M, N, K, compute_units, &sp, nullptr);
+  if (rc) return rc;
+  if (workgroup < 0 || (unsigned)workgroup >= sp.grid)
+    return fail(RL_ERR_INVALID_ARG, "workgroup %d out of range (grid %u)", workgroup, sp.grid);
+  // exactly what a workgroup of the kernel does with its (logical) index
+  unsigned unit = sk_unit_at(sp, sk_virtual_start(sp, (unsigned)workgroup));
+  const unsigned end = sk_unit_at(sp, sk_virtual_start(sp, (unsigned)workgroup + 1));
+  int n = 0;
+  while (unit < end) {
+    const sk_segment seg = sk_segment_at(sp, unit, end);
+    unit += seg.ke - seg.kb;
+    if (n < capacity) {
+      rl_streamk_segment& o = out[n];
+      o.tile_class = (int)seg.cls; o.tile = (int)seg.tile; o.tile_m = (int)seg.tile_m; o.tile_n = (int)seg.tile_n;
+      o.k_begin = (int)seg.kb; o.k_end = (int)seg.ke;
+      o.pieces = 1; o.first_workgroup = workgroup; o.slot = -1;
+      if (seg.kb != 0 || seg.ke != sp.kt) {
+        const unsigned first_wg = sk_owner(sp, seg.first_unit);
+        o.first_workgroup = (int)first_wg;
+        o.pieces = (int)(sk_owner(sp, seg.first_unit + sp.kt - 1) - first_wg + 1);
+        o.slot = 2 * workgroup + (seg.kb == 0 ? 1 : 0);
+      }
+    }
+    ++n;
+  }
+  *count = n;
   return RL_OK;
 }
 

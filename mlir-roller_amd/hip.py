@@ -61,7 +61,20 @@ class DeviceProps(C.Structure):
 class _GemmConfigC(C.Structure):
     _fields_ = [(n, C.c_int) for n in (
         "bm", "bn", "bk", "wm", "wn", "mi", "stages", "pad_a", "pad_b", "vec", "edge", "swz",
-        "group", "accum", "direct", "trans_b")]
+        "group", "accum", "direct", "trans_b", "streamk")]
+
+
+class StreamKSchedule(C.Structure):
+    """``rl_streamk_schedule``: how a stream-K configuration splits one problem."""
+    _fields_ = [("grid", C.c_int), ("k_steps", C.c_int), ("tiles", C.c_int), ("tile_rows", C.c_int), ("tile_cols", C.c_int),
+                ("units", C.c_long), ("cost", C.c_long), ("class_tiles", C.c_int * 4), ("class_cost", C.c_int * 4),
+                ("workspace_bytes", C.c_size_t), ("counter_bytes", C.c_size_t)]
+
+
+class StreamKSegment(C.Structure):
+    """``rl_streamk_segment``: one run of K steps of one tile."""
+    _fields_ = [(n, C.c_int) for n in ("tile_class", "tile", "tile_m", "tile_n", "k_begin", "k_end", "pieces",
+                                       "first_workgroup", "slot")]
 
 
 @dataclass(frozen=True)
@@ -84,6 +97,7 @@ class GemmConfig:
     accum: int = 0
     direct: int = 0
     trans_b: int = 0
+    streamk: int = 0
 
     def to_c(self) -> _GemmConfigC:
         return _GemmConfigC(*(getattr(self, f.name) for f in fields(self)))
@@ -105,7 +119,8 @@ class GemmConfig:
     def tag(self) -> str:
         return (f"b{self.bm}x{self.bn}x{self.bk}_w{self.wm}x{self.wn}_mi{self.mi}_s{self.stages}"
                 f"_p{self.pad_a}.{self.pad_b}_v{self.vec}_e{self.edge}_z{self.swz}.{self.group}"
-                f"_a{self.accum}" + ("_d1" if self.direct else "") + ("_tb" if self.trans_b else ""))
+                f"_a{self.accum}" + ("_d1" if self.direct else "") + ("_tb" if self.trans_b else "")
+                + (f"_sk{self.streamk}" if self.streamk else ""))
 
     MAX_STAGES = 5
 
@@ -121,7 +136,8 @@ def build_library(verbose: bool = False) -> Path:
     cmd = [
         "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
         "-D__HIP_PLATFORM_AMD__", f"-I{ROCM / 'include'}", f"-I{REPO_ROOT / 'include'}",
-        f'-DRL_TEMPLATE_PATH="{template}"', str(CSRC_DIR / "roller_hip.cpp"),
+        f'-DRL_TEMPLATE_PATH="{template}"', f'-DRL_SK_DECODE_PATH="{CSRC_DIR / "gemm_sk_decode.inc"}"',
+        f"-I{CSRC_DIR}", str(CSRC_DIR / "roller_hip.cpp"),
         "-o", str(LIB_PATH), f"-L{ROCM / 'lib'}", "-lamdhip64", "-lhiprtc",
         f"-Wl,-rpath,{ROCM / 'lib'}",
     ]
@@ -169,9 +185,14 @@ _SIGNATURES = {
     "rl_gemm_plan_lds_bytes": ([C.c_void_p], C.c_int),
     "rl_gemm_plan_lds_limit": ([C.c_void_p], C.c_int),
     "rl_gemm_plan_threads": ([C.c_void_p], C.c_int),
+    "rl_gemm_plan_build_log": ([C.c_void_p], C.c_char_p),
     "rl_gemm_plan_resources": ([C.c_void_p] + [C.POINTER(C.c_int)] * 5, C.c_int),
     "rl_gemm_plans_clear": ([], C.c_int),
     "rl_gemm_plan_launch": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p], C.c_int),
+    "rl_gemm_plan_workspace_bytes": ([C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)], C.c_int),
+    "rl_gemm_plan_launch_ws": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_size_t, C.c_void_p], C.c_int),
+    "rl_gemm_streamk_schedule": ([C.POINTER(_GemmConfigC)] + [C.c_int] * 4 + [C.POINTER(StreamKSchedule)], C.c_int),
+    "rl_gemm_streamk_segments": ([C.POINTER(_GemmConfigC)] + [C.c_int] * 5 + [C.POINTER(StreamKSegment), C.c_int, C.POINTER(C.c_int)], C.c_int),
     "rl_gemm_f32": ([C.POINTER(_GemmConfigC), C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p], C.c_int),
 }
 
@@ -560,13 +581,47 @@ class GemmPlan:
         check(lib().rl_gemm_plan_resources(self.handle, *[C.byref(v) for v in vals]))
         return dict(zip(("vgprs", "agprs", "sgprs", "spilled", "scratch_bytes"), (v.value for v in vals)))
 
+    def build_log(self) -> str:
+        """What hiprtc printed for this kernel ("" if nothing, or if it came from the disk cache)."""
+        return (lib().rl_gemm_plan_build_log(self.handle) or b"").decode(errors="replace")
+
+    def workspace_bytes(self, M: int, N: int, K: int) -> tuple[int, int]:
+        """(workspace bytes, of which arrival counters that must start at zero) that a launch of this
+        plan on an M x N x K problem needs; (0, 0) unless the plan is a stream-K one."""
+        total, counters = C.c_size_t(), C.c_size_t()
+        check(lib().rl_gemm_plan_workspace_bytes(self.handle, M, N, K, C.byref(total), C.byref(counters)))
+        return total.value, counters.value
+
     def launch(self, A, B, Cm, M: int, N: int, K: int, lda: Optional[int] = None,
-               ldb: Optional[int] = None, ldc: Optional[int] = None, stream=None) -> None:
+               ldb: Optional[int] = None, ldc: Optional[int] = None, stream=None, workspace=None) -> None:
+        """Enqueues the GEMM.  ``workspace`` (a ``DeviceArray``; stream-K plans only) replaces the
+        workspace that the library keeps per stream."""
         ptr = _address
         width_b = K if self.cfg.trans_b else N
-        check(lib().rl_gemm_plan_launch(self.handle, ptr(A), ptr(B), ptr(Cm), M, N, K,
-                                        K if lda is None else lda, width_b if ldb is None else ldb,
-                                        N if ldc is None else ldc, _stream_handle(stream)))
+        dims = (M, N, K, K if lda is None else lda, width_b if ldb is None else ldb, N if ldc is None else ldc)
+        if workspace is None:
+            check(lib().rl_gemm_plan_launch(self.handle, ptr(A), ptr(B), ptr(Cm), *dims, _stream_handle(stream)))
+        else:
+            check(lib().rl_gemm_plan_launch_ws(self.handle, ptr(A), ptr(B), ptr(Cm), *dims, ptr(workspace),
+                                               workspace.nbytes, _stream_handle(stream)))
+
+
+def streamk_schedule(cfg: GemmConfig, M: int, N: int, K: int, compute_units: int = 256) -> StreamKSchedule:
+    """How ``cfg`` (a stream-K configuration) splits an M x N x K problem; host arithmetic, no GPU."""
+    out, c = StreamKSchedule(), cfg.to_c()
+    check(lib().rl_gemm_streamk_schedule(C.byref(c), M, N, K, compute_units, C.byref(out)))
+    return out
+
+
+def streamk_segments(cfg: GemmConfig, M: int, N: int, K: int, workgroup: int, compute_units: int = 256) -> list:
+    """The segments that (logical) workgroup ``workgroup`` of a stream-K launch works, in order."""
+    c, count = cfg.to_c(), C.c_int()
+    buf = (StreamKSegment * 64)()
+    check(lib().rl_gemm_streamk_segments(C.byref(c), M, N, K, compute_units, workgroup, buf, 64, C.byref(count)))
+    if count.value > 64:
+        buf = (StreamKSegment * count.value)()
+        check(lib().rl_gemm_streamk_segments(C.byref(c), M, N, K, compute_units, workgroup, buf, count.value, C.byref(count)))
+    return [buf[i] for i in range(count.value)]
 
 
 def gemm_f32(cfg: GemmConfig, A, B, Cm, M: int, N: int, K: int, lda=None, ldb=None, ldc=None,

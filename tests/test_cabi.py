@@ -41,7 +41,7 @@ def test_config_struct_agrees_in_header_binding_and_documented_stub():
     in_header = [name for decl in re.findall(r"\bint\s+([a-z_,\s]+);", struct) for name in re.findall(r"[a-z_]+", decl)]
     in_binding = [name for name, _ in hip._GemmConfigC._fields_]
     in_dataclass = [f.name for f in __import__("dataclasses").fields(GemmConfig)]
-    assert in_header == in_binding == in_dataclass and in_header[-2:] == ["direct", "trans_b"]
+    assert in_header == in_binding == in_dataclass and in_header[-3:] == ["direct", "trans_b", "streamk"]
     # the binding stubs that the repository's documents show to maintainers of the reference
     docs = [p.read_text() for p in sorted(ROOT.glob("*.md"))]
     doc = next(d for d in docs if "class GemmConfig(C.Structure)" in d)
@@ -55,8 +55,10 @@ def test_config_struct_agrees_in_header_binding_and_documented_stub():
 
 
 def test_template_source_is_embedded_verbatim(hip_lib):
-    on_disk = (ROOT / "mlir-roller_amd" / "csrc" / "gemm_f32_mfma.hip").read_text()
-    assert hip.template_source() == on_disk
+    # what the JIT compiles: the work decomposition of the stream-K variant, then the template
+    csrc = ROOT / "mlir-roller_amd" / "csrc"
+    on_disk = (csrc / "gemm_f32_mfma.hip").read_text()
+    assert hip.template_source() == (csrc / "gemm_sk_decode.inc").read_text() + "\n" + on_disk
     assert 'extern "C" __global__' in on_disk and "gemm_kernel" in on_disk
 
 
