@@ -81,10 +81,9 @@ typedef struct rl_gemm_config {
                       pads the K-contiguous rows of its LDS tile like pad_a                   */
   int streamk;     /* 0: one workgroup per tile of C, grid (ceil(N/bn), ceil(M/bm)) as at src/roller.py:536.
                       1..8: a fixed grid of that many workgroups per CU; each works an equal share of all
-                      (tile, K step) units, tiles whose K range is split are summed in K order through a
-                      workspace, and (with edge) edge tiles skip the MFMA blocks outside the matrix.  Stands
-                      in for what the reference gets from ranking tilings by rounds of blocks (num_wave,
-                      src/analyze.py:164-166).  Needs stages=3                                     */
+                      (tile, K step) units, and tiles whose K range is split are summed in K order through
+                      a workspace.  Stands in for what the reference gets from ranking tilings by rounds of
+                      blocks (num_wave, src/analyze.py:164-166).  Needs stages=3                     */
 } rl_gemm_config;
 
 /* How a stream-K configuration splits one problem (rl_gemm_streamk_schedule). */
@@ -92,16 +91,13 @@ typedef struct rl_streamk_schedule {
   int grid;             /* workgroups launched */
   int k_steps;          /* K steps per tile */
   int tiles, tile_rows, tile_cols;
-  long units;           /* tiles * k_steps */
-  long cost;            /* sum over all units of their class cost; every workgroup gets cost / grid */
-  int class_tiles[4];   /* tiles per class: interior, right column, bottom row, corner */
-  int class_cost[4];    /* cost of one K step per class (MFMA blocks of the busiest wave, with a floor) */
+  long units;           /* tiles * k_steps; every workgroup gets units / grid of them, give or take one */
   size_t workspace_bytes, counter_bytes;
 } rl_streamk_schedule;
 
 /* One run of K steps of one tile, as a workgroup of a stream-K launch works it. */
 typedef struct rl_streamk_segment {
-  int tile_class, tile, tile_m, tile_n;
+  int tile, tile_m, tile_n;  /* tile number in walk order (its arrival counter), tile row and column */
   int k_begin, k_end;        /* K steps [k_begin, k_end) of the tile */
   int pieces;                /* workgroups that share the tile (1: this segment is the whole tile) */
   int first_workgroup;       /* the one with the tile's first K steps; the pieces follow in workgroup order */

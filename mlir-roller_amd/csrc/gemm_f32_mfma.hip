@@ -52,9 +52,8 @@
 //               (gemm_sk_decode.inc).  A tile whose K range is split over workgroups is summed through
 //               a workspace: every piece is stored there, an arrival counter per tile tells the last
 //               piece in, and that workgroup adds the pieces in K order and writes C -- the same
-//               order whoever arrives last, so results are bit-identical from run to run.  With EDGE,
-//               tiles on the right and bottom edges skip the MFMA blocks that lie outside the matrix
-//               (their K steps then cost less, which the split accounts for).  Needs STAGES == 3.
+//               order whoever arrives last, so results are bit-identical from run to run.  Needs
+//               STAGES == 3.
 //   TRANS_B     1 = the second operand is given transposed, Bt[N][ldb >= K] (K contiguous, the
 //               layout in which the policy models both inputs, /root/reference/src/analyze.py:33-41).
 //               Its tile then sits in LDS like the A tile ([BN][BK+PAD_B], swizzled under DIRECT)
@@ -179,6 +178,8 @@
 #define A_PER_T ((A_UNITS + NT - 1) / NT)
 #define B_PER_T ((B_UNITS + NT - 1) / NT)
 #define OOB_OFFSET 0x80000000u
+/* cache policy operand of a buffer access: sc0 (bit 0) and sc1 (bit 4) together = coherent across the whole system */
+#define SK_COHERENT 0x11
 /* DIRECT: 16-byte chunks per A row; A rows per 256 bytes of LDS (the 64 banks that a 128-bit read
  * of 16 lanes must cover without collision); the swizzle period.  Rows that start at the same
  * offset within a 256-byte window get their chunks XOR-ed with distinct values, so the 16 lanes
@@ -435,32 +436,22 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     wg = xcd < tall ? xcd * per + loc : tall * per + (xcd - tall) * (per - 1) + loc;
   }
 #endif
-  unsigned sk_unit = sk_unit_at(sk, sk_virtual_start(sk, wg));
-  const unsigned sk_end = sk_unit_at(sk, sk_virtual_start(sk, wg + 1));
+  unsigned sk_unit = sk_first_unit(sk, wg);
+  const unsigned sk_end = sk_first_unit(sk, wg + 1);
   for (bool again = false; sk_unit < sk_end; again = true) {
   const sk_segment seg = sk_segment_at(sk, sk_unit, sk_end);
   sk_unit += seg.ke - seg.kb;
   const int tile_m = (int)seg.tile_m, tile_n = (int)seg.tile_n;
   const int kb = (int)seg.kb;                       // first K step of the segment
-  const bool skip_blocks = EDGE && seg.cls != 0;    // an edge tile that leaves out the MFMA blocks outside the matrix
   if (again) __syncthreads();                       // every wave is done with the LDS tiles of the previous segment
 #else
   const int nbm = (M + BM - 1) / BM, nbn = (N + BN - 1) / BN;
   int tile_m, tile_n;
   if (!tile_of_workgroup(nbm, nbn, tile_m, tile_n)) return;
   constexpr int kb = 0;
-  constexpr bool skip_blocks = false;
   {
 #endif
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  // MFMA blocks of this wave that reach into the matrix (all of them unless blocks are skipped)
-  const int tm_act = !skip_blocks ? TM : (M - m0 - wm0 <= 0 ? 0 : (M - m0 - wm0 + MI - 1) / MI < TM ? (M - m0 - wm0 + MI - 1) / MI : TM);
-  // (a B read feeds the blocks of a segment column by column -- block e owns every w-th column -- so
-  // along N whole segments stay or go: tn_act is the end of the last segment that reaches into the matrix)
-  const int tn_need = N - n0 - wn0 <= 0 ? 0 : (N - n0 - wn0 + MI - 1) / MI;
-  const int tn_act = !skip_blocks ? TN
-                     : tn_need <= 4 * NSEG4 ? (tn_need + 3) / 4 * 4
-                     : (HAS_SEG2 && tn_need <= 4 * NSEG4 + 2) ? 4 * NSEG4 + 2 : TN;
 
   // ---- global -> register staging: per-thread loop-invariant offsets ----
   unsigned a_goff[A_PER_T], b_goff[B_PER_T];
@@ -682,19 +673,13 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     }
 #endif
   };
-  // SKIP (a compile-time 0/1): leave out the blocks at or beyond (tm_act, tn_act) -- a wave-uniform
-  // test per row and per block, which costs scalar branches and the static interleave, so only the
-  // edge tiles of the stream-K variant take this form.
-  auto mfma_frags = [&](auto skip, const frag_t& f, int t0 = 0, int t1 = 4) __attribute__((always_inline)) {
-    constexpr bool SKIP = decltype(skip)::value;
+  auto mfma_frags = [&](const frag_t& f, int t0 = 0, int t1 = 4) __attribute__((always_inline)) {
 #pragma unroll
     for (int t = t0; t < t1; ++t)
 #pragma unroll
-      for (int bi = 0; bi < TM; ++bi) {
-        if (SKIP && bi >= tm_act) continue;
+      for (int bi = 0; bi < TM; ++bi)
 #pragma unroll
         for (int bj = 0; bj < TN; ++bj) {
-          if (SKIP && bj >= tn_act) continue;
 #if TRANS_B
           const float bval = f.b[bj][t];
 #else
@@ -702,13 +687,11 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
           acc[bi][bj] = MFMA(f.a[bi][t], bval, acc[bi][bj]);
         }
-      }
   };
 
   // ---- main loop ----
 #if STAGES >= 3
-  auto main_loop = [&](auto skip) __attribute__((always_inline)) {
-    constexpr bool SKIP = decltype(skip)::value;
+  if (KT > 0) {
     // Software pipeline.  At the top of step kt: tile kt is in its LDS buffer, its first fragment
     // round is already in registers, and the staging registers hold tile kt+1 (loaded during step
     // kt-1).  Within the step each fragment round is read while the previous one is in the MFMA
@@ -757,34 +740,31 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
-        mfma_frags(skip, fr[(P + r) & 1]);
+        mfma_frags(fr[(P + r) & 1]);
       }
       // the last round is split around the barrier: its first half covers the LDS writes of
       // tile kt+1 and the global loads of tile kt+2, its second half the first reads of tile kt+1
       // (DIRECT: one quarter before the barrier, three after it, which leaves room to issue the
       // loads of tile kt+2 behind every second MFMA instead of every one: measured 0.3-0.8 % faster)
 #if DIRECT
-      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 0, 1);
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 1);
       // Tile kt+1 was requested LDS_BUFS-1 steps ago, straight into the next buffer; once every
       // wave's part has landed (the requests for later tiles may still be in flight) and all have
       // met, buffer `cur` is free again and takes tile kt+LDS_BUFS.
 #if SCHED
-      if constexpr (!SKIP) {
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
       // the barrier (and the wait for the LDS reads that comes with it) stays behind the MFMAs above:
       // left to float, it lands right behind the last read and the wave sits out that read's latency
       interleave_with_mfma<G / 4, 0, 0x100>();
       __builtin_amdgcn_sched_barrier(0);
-      }
 #endif
       WAIT_VMCNT((LDS_BUFS - 2) * LOADS_PER_TILE);
       __syncthreads();
       read_frags(fr[(P + SUPERS) & 1], nxt, 0);
       fetch_direct(ktail, kt + LDS_BUFS, cur);
-      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 1, 4);
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 1, 4);
 #if SCHED
-      if constexpr (!SKIP) {
       {
         constexpr int REST = 3 * G / 4, PAIRED = R < REST ? R : REST, LEFT = REST - PAIRED;
         interleave_with_mfma<PAIRED, R, 0x100>();
@@ -794,27 +774,22 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
           interleave_with_mfma<LEFT, L, 0x020>();
         }
       }
-      }
 #endif
 #else
-      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 0, 2);
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 0, 2);
       stash(nxt);
       fetch(ktail, kt + 2);
 #if SCHED
-      if constexpr (!SKIP) {
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
       interleave_with_mfma<G / 4, W, 0x200>();
       interleave_with_mfma<G / 2 - G / 4, L, 0x020>();
-      }
 #endif
       __syncthreads();
       read_frags(fr[(P + SUPERS) & 1], nxt, 0);
-      mfma_frags(skip, fr[(P + SUPERS - 1) & 1], 2, 4);
+      mfma_frags(fr[(P + SUPERS - 1) & 1], 2, 4);
 #if SCHED
-      if constexpr (!SKIP) {
       interleave_with_mfma<G / 2, R, 0x100>();
-      }
 #endif
 #endif
     };
@@ -824,14 +799,12 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) {
         read_frags(fr[(P + r + 1) & 1], cur, (r + 1) * KSUPER);
-        mfma_frags(skip, fr[(P + r) & 1]);
+        mfma_frags(fr[(P + r) & 1]);
       }
-      mfma_frags(skip, fr[(P + SUPERS - 1) & 1]);
+      mfma_frags(fr[(P + SUPERS - 1) & 1]);
 #if SCHED
-      if constexpr (!SKIP) {
 #pragma unroll
       for (int r = 0; r + 1 < SUPERS; ++r) interleave_with_mfma<G, R, 0x100>();
-      }
 #endif
 #if DIRECT
       WAIT_VMCNT(0);  // the (empty) requests for the tiles past the end have drained
@@ -864,13 +837,6 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (; kt + 1 < pipelined; kt += 2) pair(int_c<0>{}, kt);
 #endif
     last_step(int_c<0>{}, int_c<0>{}, pipelined);
-  };
-  if (KT > 0) {
-#if STREAMK && EDGE
-    if (skip_blocks) main_loop(int_c<1>{}); else main_loop(int_c<0>{});
-#else
-    main_loop(int_c<0>{});
-#endif
   }
 #else
   static_assert(!DIRECT, "DIRECT belongs to the pipelined loop");
@@ -879,7 +845,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     for (int kk = 0; kk < BK; kk += KSUPER) {
       frag_t f;
       read_frags(f, stage, kk);
-      mfma_frags(int_c<0>{}, f);
+      mfma_frags(f);
     }
   };
   if (KT > 0) {
@@ -915,11 +881,20 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   // the tile's counter at pieces - 1 was last: it adds all pieces up in K order, its own included
   // (read back, so the sum is formed the same way whoever comes last), stores C and clears the
   // counter for the next launch.
+  //
+  // Pieces are written and read with the sc0 sc1 cache policy: stores go through the caches to
+  // memory and loads come from there, past whatever this XCD's L2 holds, so a piece needs no
+  // cache-wide write-back on the writer's side and no invalidate on the reader's (either of which would
+  // empty the L2 that the other workgroups of the XCD share their operand panels through -- measured:
+  // with fences the split cost more than it saved).  A writer waits until its stores have been
+  // acknowledged (vmcnt 0) before its workgroup is counted in; the reader only reads once it has
+  // seen the count.
   bool store_c = true;
   if (seg.kb != 0 || seg.ke != sk.kt) {
     constexpr int CHUNKS = ACC_REGS / 4;            // 16-byte chunks per MFMA block and lane
-    const unsigned first_wg = sk_owner(sk, seg.first_unit);
-    const unsigned pieces = sk_owner(sk, seg.first_unit + sk.kt - 1) - first_wg + 1;
+    const unsigned tile_unit = seg.tile * sk.kt;     // unit number of the tile's first K step
+    const unsigned first_wg = sk_owner(sk, tile_unit);
+    const unsigned pieces = sk_owner(sk, tile_unit + sk.kt - 1) - first_wg + 1;
     const unsigned my_slot = 2 * wg + (seg.kb == 0 ? 1 : 0);
     {
       const __amdgpu_buffer_rsrc_t wr = make_rsrc(sk_slots + (long)my_slot * (BM * BN), (long)BM * BN * 4);
@@ -930,19 +905,18 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
           for (int c = 0; c < CHUNKS; ++c) {
             const v4f v = {acc[bi][bj][4 * c], acc[bi][bj][4 * c + 1], acc[bi][bj][4 * c + 2], acc[bi][bj][4 * c + 3]};
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), wr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), wr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, SK_COHERENT);
           }
     }
-    // make the piece visible to the whole device, then count this workgroup in
-    __threadfence();
+    // the piece has arrived in memory; then count this workgroup in
+    WAIT_VMCNT(0);
     __syncthreads();
     if (tid == 0)
-      lds[0] = __builtin_bit_cast(float, __hip_atomic_fetch_add(&sk_arrivals[seg.tile], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT));
+      lds[0] = __builtin_bit_cast(float, __hip_atomic_fetch_add(&sk_arrivals[seg.tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     __syncthreads();
     const unsigned before = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(unsigned, lds[0]));
     store_c = before == pieces - 1;
     if (store_c) {
-      __threadfence();   // the other pieces, as their workgroups released them
       auto add_piece = [&](auto is_first, unsigned slot) __attribute__((always_inline)) {
         const __amdgpu_buffer_rsrc_t rr = make_rsrc(sk_slots + (long)slot * (BM * BN), (long)BM * BN * 4);
 #pragma unroll
@@ -951,7 +925,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
           for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
             for (int c = 0; c < CHUNKS; ++c) {
-              const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, 0));
+              const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, SK_COHERENT));
 #pragma unroll
               for (int e = 0; e < 4; ++e) acc[bi][bj][4 * c + e] = decltype(is_first)::value ? v[e] : acc[bi][bj][4 * c + e] + v[e];
             }

@@ -416,80 +416,29 @@ sk_div make_div(unsigned d) {
   return out;
 }
 
-// Cost of one K step of an edge tile relative to the MFMA blocks it keeps: below a quarter of a full
-// tile's blocks a step is bounded by its loads and barrier, not by its MFMAs.  Overridable for
-// experiments (percent of a full tile's cost).
-unsigned min_step_cost(unsigned full) {
-  static const int percent = [] {
-    const char* e = getenv("ROLLER_SK_MIN_COST_PERCENT");
-    const int v = e ? atoi(e) : 25;
-    return v < 1 ? 1 : (v > 100 ? 100 : v);
-  }();
-  const unsigned m = (full * (unsigned)percent + 99) / 100;
-  return m < 1 ? 1 : m;
-}
-
-// Fills *p for cfg on an M x N x K problem with `compute_units` CUs.  Edge classes exist when the
-// kernel predicates edges (cfg.edge) and the busiest wave of such a tile keeps fewer MFMA blocks than
-// a full tile has.  The grid is cfg.streamk workgroups per CU, cut down where the problem is too
-// small to give every workgroup one full-cost K step (the decoding relies on no share being empty).
+// Fills *p for cfg on an M x N x K problem with `compute_units` CUs.  The grid is cfg.streamk
+// workgroups per CU, cut down to one K step per workgroup where the problem is smaller than that
+// (the decoding relies on no share being empty).
 int sk_make_params(const rl_gemm_config& c, int M, int N, int K, int compute_units, sk_params* p, unsigned* tiles) {
   if (!c.streamk) return fail(RL_ERR_INVALID_ARG, "not a stream-K configuration");
   if (M <= 0 || N <= 0 || K <= 0) return fail(RL_ERR_INVALID_ARG, "stream-K needs M, N, K > 0 (M=%d N=%d K=%d)", M, N, K);
   if (compute_units <= 0) return fail(RL_ERR_INVALID_ARG, "compute_units must be positive");
   const unsigned long nbm = ((unsigned long)M + c.bm - 1) / c.bm, nbn = ((unsigned long)N + c.bn - 1) / c.bn;
   const unsigned long kt = ((unsigned long)K + c.bk - 1) / c.bk;
-  const unsigned tm = c.wm / c.mi, tn = c.wn / c.mi, full = tm * tn;
-  const unsigned mrem = (unsigned)(M - (long)(nbm - 1) * c.bm), nrem = (unsigned)(N - (long)(nbn - 1) * c.bn);
-  // MFMA blocks that the wave at the tile's origin (the busiest one) keeps: block rows one by one, block
-  // columns by whole read segments (four blocks, then two, then one), as the kernel skips them
-  auto block_rows = [&](unsigned valid) {
-    const unsigned b = (valid + c.mi - 1) / c.mi;
-    return b < tm ? b : tm;
-  };
-  auto block_cols = [&](unsigned valid) {
-    const unsigned b = (valid + c.mi - 1) / c.mi, fours = tn / 4 * 4;
-    if (b <= fours) return (b + 3) / 4 * 4;
-    if ((tn % 4) / 2 && b <= fours + 2) return fours + 2;
-    return tn;
-  };
-  const unsigned floor_cost = min_step_cost(full);
-  auto cost = [&](unsigned rows, unsigned cols) {
-    const unsigned b = block_rows(rows) * block_cols(cols);
-    return b < floor_cost ? floor_cost : b;
-  };
-  const unsigned w_right = cost(c.bm, nrem), w_bottom = cost(mrem, c.bn), w_corner = cost(mrem, nrem);
-  const bool has_r = c.edge && nrem < (unsigned)c.bn && w_right < full;
-  const bool has_b = c.edge && mrem < (unsigned)c.bm && w_bottom < full;
-  const unsigned long nim = nbm - (has_b ? 1 : 0), nin = nbn - (has_r ? 1 : 0);
-  const unsigned long count[4] = {nim * nin, has_r ? nim : 0, has_b ? nin : 0, (has_r && has_b) ? 1ul : 0ul};
-  // a corner next to only one skipped edge belongs to that edge's class
-  const unsigned w[4] = {full, w_right, w_bottom, w_corner};
-  unsigned long u = 0, v = 0, t = 0, ub[5], vb[5], tb[4];
-  for (int k = 0; k < 4; ++k) {
-    ub[k] = u; vb[k] = v; tb[k] = t;
-    u += count[k] * kt; v += count[k] * kt * w[k]; t += count[k];
-  }
-  ub[4] = u; vb[4] = v;
-  if (v >= 0x7fffffffUL || u >= 0x7fffffffUL || nbm > 0xffffffUL || nbn > 0xffffffUL)
-    return fail(RL_ERR_INVALID_ARG, "problem too large for the 32-bit arithmetic of the stream-K split (%lu units of cost %lu)", u, v);
+  const unsigned long units = nbm * nbn * kt;
+  if (units >= 0x7fffffffUL || nbm > 0xffffffUL || nbn > 0xffffffUL)
+    return fail(RL_ERR_INVALID_ARG, "problem too large for the 32-bit arithmetic of the stream-K split (%lu units)", units);
   unsigned long grid = (unsigned long)compute_units * c.streamk;
-  if (grid > v / full) grid = v / full;     // every share at least one full-cost K step: no share is empty
-  if (grid < 1) grid = 1;
+  if (grid > units) grid = units;
   memset(p, 0, sizeof *p);
-  p->grid = (unsigned)grid; p->q = (unsigned)(v / grid); p->r = (unsigned)(v % grid); p->kt = (unsigned)kt;
-  p->nbm = (unsigned)nbm; p->nbn = (unsigned)nbn; p->nim = (unsigned)nim; p->nin = (unsigned)nin;
+  p->grid = (unsigned)grid; p->q = (unsigned)(units / grid); p->r = (unsigned)(units % grid); p->kt = (unsigned)kt;
+  p->nbm = (unsigned)nbm; p->nbn = (unsigned)nbn;
   p->group = (c.swz & 2) ? (unsigned)(c.group > 0 ? c.group : 1) : 1u;
-  p->rows_last = (unsigned)(nim % p->group);
-  p->w0 = w[0]; p->w1 = w[1]; p->w2 = w[2]; p->w3 = w[3];
-  p->u1 = (unsigned)ub[1]; p->u2 = (unsigned)ub[2]; p->u3 = (unsigned)ub[3]; p->u4 = (unsigned)ub[4];
-  p->v1 = (unsigned)vb[1]; p->v2 = (unsigned)vb[2]; p->v3 = (unsigned)vb[3];
-  p->t1 = (unsigned)tb[1]; p->t2 = (unsigned)tb[2]; p->t3 = (unsigned)tb[3];
+  p->rows_last = (unsigned)(nbm % p->group);
   p->d_kt = make_div(p->kt); p->d_q = make_div(p->q); p->d_q1 = make_div(p->q + 1);
-  p->d_width = make_div(p->group * (p->nin ? p->nin : 1)); p->d_group = make_div(p->group);
+  p->d_width = make_div(p->group * p->nbn); p->d_group = make_div(p->group);
   p->d_rows_last = make_div(p->rows_last ? p->rows_last : 1);
-  p->d_w0 = make_div(w[0]); p->d_w1 = make_div(w[1]); p->d_w2 = make_div(w[2]); p->d_w3 = make_div(w[3]);
-  if (tiles) *tiles = (unsigned)t;
+  if (tiles) *tiles = (unsigned)(nbm * nbn);
   return RL_OK;
 }
 
@@ -1030,13 +979,7 @@ int rl_gemm_streamk_schedule(const rl_gemm_config* cfg, int M, int N, int K, int
   out->tiles = (int)tiles;
   out->tile_rows = (int)sp.nbm;
   out->tile_cols = (int)sp.nbn;
-  out->units = (long)sp.u4;
-  out->cost = (long)sp.grid * sp.q + sp.r;
-  const unsigned first[5] = {0u, sp.u1, sp.u2, sp.u3, sp.u4}, w[4] = {sp.w0, sp.w1, sp.w2, sp.w3};
-  for (int k = 0; k < 4; ++k) {
-    out->class_tiles[k] = (int)((first[k + 1] - first[k]) / sp.kt);
-    out->class_cost[k] = (int)w[k];
-  }
+  out->units = (long)sp.grid * sp.q + sp.r;
   out->workspace_bytes = sk_workspace_bytes(*cfg, sp, tiles);
   out->counter_bytes = sk_counter_bytes(tiles);
   return RL_OK;
@@ -1053,21 +996,21 @@ int rl_gemm_streamk_segments(const rl_gemm_config* cfg, int M, int N, int K, int
   if (workgroup < 0 || (unsigned)workgroup >= sp.grid)
     return fail(RL_ERR_INVALID_ARG, "workgroup %d out of range (grid %u)", workgroup, sp.grid);
   // exactly what a workgroup of the kernel does with its (logical) index
-  unsigned unit = sk_unit_at(sp, sk_virtual_start(sp, (unsigned)workgroup));
-  const unsigned end = sk_unit_at(sp, sk_virtual_start(sp, (unsigned)workgroup + 1));
+  unsigned unit = sk_first_unit(sp, (unsigned)workgroup);
+  const unsigned end = sk_first_unit(sp, (unsigned)workgroup + 1);
   int n = 0;
   while (unit < end) {
     const sk_segment seg = sk_segment_at(sp, unit, end);
     unit += seg.ke - seg.kb;
     if (n < capacity) {
       rl_streamk_segment& o = out[n];
-      o.tile_class = (int)seg.cls; o.tile = (int)seg.tile; o.tile_m = (int)seg.tile_m; o.tile_n = (int)seg.tile_n;
+      o.tile = (int)seg.tile; o.tile_m = (int)seg.tile_m; o.tile_n = (int)seg.tile_n;
       o.k_begin = (int)seg.kb; o.k_end = (int)seg.ke;
       o.pieces = 1; o.first_workgroup = workgroup; o.slot = -1;
       if (seg.kb != 0 || seg.ke != sp.kt) {
-        const unsigned first_wg = sk_owner(sp, seg.first_unit);
+        const unsigned first_wg = sk_owner(sp, seg.tile * sp.kt);
         o.first_workgroup = (int)first_wg;
-        o.pieces = (int)(sk_owner(sp, seg.first_unit + sp.kt - 1) - first_wg + 1);
+        o.pieces = (int)(sk_owner(sp, seg.tile * sp.kt + sp.kt - 1) - first_wg + 1);
         o.slot = 2 * workgroup + (seg.kb == 0 ? 1 : 0);
       }
     }

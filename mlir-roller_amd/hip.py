@@ -67,13 +67,12 @@ class _GemmConfigC(C.Structure):
 class StreamKSchedule(C.Structure):
     """``rl_streamk_schedule``: how a stream-K configuration splits one problem."""
     _fields_ = [("grid", C.c_int), ("k_steps", C.c_int), ("tiles", C.c_int), ("tile_rows", C.c_int), ("tile_cols", C.c_int),
-                ("units", C.c_long), ("cost", C.c_long), ("class_tiles", C.c_int * 4), ("class_cost", C.c_int * 4),
-                ("workspace_bytes", C.c_size_t), ("counter_bytes", C.c_size_t)]
+                ("units", C.c_long), ("workspace_bytes", C.c_size_t), ("counter_bytes", C.c_size_t)]
 
 
 class StreamKSegment(C.Structure):
     """``rl_streamk_segment``: one run of K steps of one tile."""
-    _fields_ = [(n, C.c_int) for n in ("tile_class", "tile", "tile_m", "tile_n", "k_begin", "k_end", "pieces",
+    _fields_ = [(n, C.c_int) for n in ("tile", "tile_m", "tile_n", "k_begin", "k_end", "pieces",
                                        "first_workgroup", "slot")]
 
 

@@ -48,7 +48,7 @@ CASES = [
     (GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2), [(256, 384, 128), (1024, 1024, 2048), (2304, 2048, 512), (128, 128, 32)]),
     # ragged in every dimension, K tail in the last piece, problems smaller than a tile
     (GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1, 0, 2), [(200, 300, 200), (130, 260, 96), (1, 4, 4), (1000, 1000, 1000), (2100, 1900, 1124)]),
-    # edge tiles that skip MFMA blocks: right column, bottom row, corner; 32x32x2 and 16x16x4; one wave along N
+    # ragged M and N with whole K steps (no K predicates in the loop); 32x32x2 and 16x16x4; one wave along N
     (GemmConfig(96, 160, 32, 48, 80, 16, 3, 0, 0, 4, 2, 3, 8, 0, 1, 0, 2), [(3000, 5000, 1536), (200, 340, 64), (96 * 3 + 24, 160 * 2 + 40, 96)]),
     (GemmConfig(96, 160, 32, 48, 80, 16, 3, 0, 0, 4, 2, 3, 8, 0, 1, 0, 1), [(1500, 2500, 768)]),
     (GemmConfig(64, 320, 32, 16, 320, 16, 3, 0, 0, 4, 2, 3, 8, 0, 1, 0, 1), [(3000, 5000, 1536), (130, 700, 64)]),
@@ -71,7 +71,7 @@ FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
 def test_streamk_matches_oracle_within_tolerance_and_exactly_on_integers(device, cfg, shape):
     M, N, K = shape
     sched = hip.streamk_schedule(cfg, M, N, K, device.compute_units)
-    say("case", cfg.tag(), shape, "grid", sched.grid, "classes", list(sched.class_tiles), list(sched.class_cost))
+    say("case", cfg.tag(), shape, "grid", sched.grid, "tiles", sched.tiles, "K steps", sched.k_steps)
     Ai, Bi = go.make_inputs(M, N, K, seed=1, distribution="integer")
     want = host_gemm(Ai, Bi)
     got = run(cfg, Ai, Bi)
