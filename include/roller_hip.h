@@ -233,6 +233,20 @@ int rl_gemm_plan_launch_ws(const rl_gemm_plan* plan, const float* A, const float
                            int M, int N, int K, int lda, int ldb, int ldc, void* workspace,
                            size_t workspace_bytes, rl_stream stream);
 
+/* rl_gemm_plan_launch for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  It calls no
+ * hipMalloc / hipFree / allocating routine on any path: a stream-K plan takes its workspace from a
+ * fixed array in device memory that is part of the library's own code object (256 KiB of arrival
+ * counters + 64 MiB of slots; every GPU the library runs on holds it until the process ends), and a
+ * launch that needs more -- more than 65536 tiles, or 2 * workgroups * bm * bn * 4 bytes beyond 64 MiB
+ * -- is refused with RL_ERR_INVALID_ARG and text.  All calls on a GPU share that one array: calls that
+ * overlap on the device (different streams) race; calls on one stream do not.  The kernels leave the
+ * counters at zero, the slots keep the last call's pieces (every call overwrites what it reads).  For a
+ * plan without streamk it is rl_gemm_plan_launch.  K == 0 writes zeros with a small fill kernel
+ * (never a memset call, so the launch may sit in a captured graph). */
+int rl_gemm_plan_launch_static(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
+                               int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream);
+
 /* The split of an M x N x K problem under a stream-K configuration on a device with `compute_units`
  * CUs, and the segments that workgroup `workgroup` works (at most `capacity` are written, *count
  * receives how many there are).  Host arithmetic only (no device needed): what the policy's cost

@@ -7,6 +7,7 @@
 // .incbin and handed to hiprtc at run time.
 
 #include "roller_hip.h"
+#include "roller_scratch.h"
 
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
@@ -479,7 +480,7 @@ int workspace_for(hipStream_t stream, size_t bytes, void** out) {
   return RL_OK;
 }
 
-enum WorkspaceKind { WS_LIBRARY, WS_CALLER };
+enum WorkspaceKind { WS_LIBRARY, WS_CALLER, WS_STATIC };
 
 // Argument checks and launch shared by the plan entry points.  A stream-K plan takes its workspace
 // from the library (one per stream) or from the caller.
@@ -525,7 +526,7 @@ int launch_plan(const rl_gemm_plan* plan, const float* A, const float* B, float*
 
   if (K == 0) {
     // no K step to hand out: C = 0 (or C unchanged when accumulating), without the kernel
-    if (!c.accum) HIP_TRY(hipMemset2DAsync(C, (size_t)ldc * 4, 0, (size_t)N * 4, (size_t)M, (hipStream_t)stream));
+    if (!c.accum) HIP_TRY(rl_scratch_zero_c(C, ldc, M, N, (hipStream_t)stream));
     return RL_OK;
   }
   sk_params sp;
@@ -534,7 +535,17 @@ int launch_plan(const rl_gemm_plan* plan, const float* A, const float* B, float*
   if (rc) return rc;
   const size_t need = sk_workspace_bytes(c, sp, tiles);
   void* ws = nullptr;
-  if (kind == WS_CALLER) {
+  // the counters sit at the front of a workspace; the static array keeps a fixed room for them
+  size_t counter_room = sk_counter_bytes(tiles);
+  if (kind == WS_STATIC) {
+    ws = rl_scratch_address(g_device.load());
+    if (!ws) return fail(RL_ERR_NO_DEVICE, "the static scratch array was not set up (rl_init)");
+    counter_room = RL_STATIC_SCRATCH_COUNTER_BYTES;
+    const size_t slots = need - sk_counter_bytes(tiles);
+    if (sk_counter_bytes(tiles) > counter_room || slots > RL_STATIC_SCRATCH_BYTES - counter_room)
+      return fail(RL_ERR_INVALID_ARG, "rl_gemm_plan_launch_static: this launch needs %zu bytes of counters and %zu bytes of slots; the static scratch array holds %u and %u (use rl_gemm_plan_launch or rl_gemm_plan_launch_ws)",
+                  sk_counter_bytes(tiles), slots, RL_STATIC_SCRATCH_COUNTER_BYTES, RL_STATIC_SCRATCH_BYTES - RL_STATIC_SCRATCH_COUNTER_BYTES);
+  } else if (kind == WS_CALLER) {
     if (!user_ws || user_ws_bytes < need)
       return fail(RL_ERR_INVALID_ARG, "stream-K launch needs a workspace of %zu bytes (rl_gemm_plan_workspace_bytes), got %zu", need, user_ws ? user_ws_bytes : (size_t)0);
     if ((uintptr_t)user_ws & 255) return fail(RL_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
@@ -544,7 +555,7 @@ int launch_plan(const rl_gemm_plan* plan, const float* A, const float* B, float*
     if (rc) return rc;
   }
   unsigned* arrivals = (unsigned*)ws;
-  float* slots = (float*)((char*)ws + sk_counter_bytes(tiles));
+  float* slots = (float*)((char*)ws + counter_room);
   void* args[] = {(void*)&A, (void*)&B, (void*)&C, &M, &N, &K, &lda, &ldb, &ldc, &slots, &arrivals, &sp};
   HIP_TRY(hipModuleLaunchKernel(plan->func, sp.grid, 1, 1, (unsigned)plan->threads, 1, 1,
                                 (unsigned)plan->lds_bytes, (hipStream_t)stream, args, nullptr));
@@ -576,6 +587,8 @@ int rl_init(int device) {
   int attr = 0;
   if (hipDeviceGetAttribute(&attr, hipDeviceAttributeMaxSharedMemoryPerBlock, device) == hipSuccess && attr > lds_limit)
     lds_limit = attr;
+  // where this device keeps the library's static scratch array (rl_gemm_plan_launch_static)
+  HIP_TRY(rl_scratch_setup(device));
   g_lds_limit = lds_limit;
   g_compute_units = prop.multiProcessorCount;
   g_device = device;
@@ -947,6 +960,11 @@ int rl_gemm_plan_launch_ws(const rl_gemm_plan* plan, const float* A, const float
                            int M, int N, int K, int lda, int ldb, int ldc, void* workspace,
                            size_t workspace_bytes, rl_stream stream) {
   return launch_plan(plan, A, B, C, M, N, K, lda, ldb, ldc, stream, WS_CALLER, workspace, workspace_bytes);
+}
+
+int rl_gemm_plan_launch_static(const rl_gemm_plan* plan, const float* A, const float* B, float* C,
+                               int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream) {
+  return launch_plan(plan, A, B, C, M, N, K, lda, ldb, ldc, stream, WS_STATIC, nullptr, 0);
 }
 
 int rl_gemm_plan_workspace_bytes(const rl_gemm_plan* plan, int M, int N, int K, size_t* bytes, size_t* counter_bytes) {

@@ -129,20 +129,27 @@ class GemmConfig:
 # --------------------------------------------------------------------------------------------
 
 def build_library(verbose: bool = False) -> Path:
-    """Compiles csrc/roller_hip.cpp into libroller_hip.so (host code; the kernel template is
-    embedded as text and compiled for gfx950 by hiprtc at run time or by ``precompile``)."""
+    """Builds libroller_hip.so: csrc/roller_hip.cpp (host code; the kernel template is embedded as text
+    and compiled for gfx950 by hiprtc at run time or by ``precompile``) and csrc/roller_scratch.hip
+    (hipcc, gfx950: the static scratch array of the launch entry point that allocates nothing)."""
     template = CSRC_DIR / "gemm_f32_mfma.hip"
-    cmd = [
-        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
-        "-D__HIP_PLATFORM_AMD__", f"-I{ROCM / 'include'}", f"-I{REPO_ROOT / 'include'}",
-        f'-DRL_TEMPLATE_PATH="{template}"', f'-DRL_SK_DECODE_PATH="{CSRC_DIR / "gemm_sk_decode.inc"}"',
-        f"-I{CSRC_DIR}", str(CSRC_DIR / "roller_hip.cpp"),
-        "-o", str(LIB_PATH), f"-L{ROCM / 'lib'}", "-lamdhip64", "-lhiprtc",
-        f"-Wl,-rpath,{ROCM / 'lib'}",
+    obj_dir = REPO_ROOT / "build"
+    obj_dir.mkdir(exist_ok=True)
+    scratch_obj = obj_dir / "roller_scratch.o"
+    cmds = [
+        ["hipcc", "--offload-arch=gfx950", "-O2", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         f"-I{CSRC_DIR}", "-c", str(CSRC_DIR / "roller_scratch.hip"), "-o", str(scratch_obj)],
+        ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-Wextra",
+         "-D__HIP_PLATFORM_AMD__", f"-I{ROCM / 'include'}", f"-I{REPO_ROOT / 'include'}",
+         f'-DRL_TEMPLATE_PATH="{template}"', f'-DRL_SK_DECODE_PATH="{CSRC_DIR / "gemm_sk_decode.inc"}"',
+         f"-I{CSRC_DIR}", str(CSRC_DIR / "roller_hip.cpp"), str(scratch_obj),
+         "-o", str(LIB_PATH), f"-L{ROCM / 'lib'}", "-lamdhip64", "-lhiprtc",
+         f"-Wl,-rpath,{ROCM / 'lib'}"],
     ]
-    if verbose:
-        print(" ".join(cmd))
-    subprocess.run(cmd, check=True)
+    for cmd in cmds:
+        if verbose:
+            print(" ".join(cmd))
+        subprocess.run(cmd, check=True)
     global _lib
     _lib = None
     return LIB_PATH
@@ -190,6 +197,7 @@ _SIGNATURES = {
     "rl_gemm_plan_launch": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p], C.c_int),
     "rl_gemm_plan_workspace_bytes": ([C.c_void_p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)], C.c_int),
     "rl_gemm_plan_launch_ws": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p, C.c_size_t, C.c_void_p], C.c_int),
+    "rl_gemm_plan_launch_static": ([C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p], C.c_int),
     "rl_gemm_streamk_schedule": ([C.POINTER(_GemmConfigC)] + [C.c_int] * 4 + [C.POINTER(StreamKSchedule)], C.c_int),
     "rl_gemm_streamk_segments": ([C.POINTER(_GemmConfigC)] + [C.c_int] * 5 + [C.POINTER(StreamKSegment), C.c_int, C.POINTER(C.c_int)], C.c_int),
     "rl_gemm_f32": ([C.POINTER(_GemmConfigC), C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 6 + [C.c_void_p], C.c_int),
@@ -593,12 +601,15 @@ class GemmPlan:
 
     def launch(self, A, B, Cm, M: int, N: int, K: int, lda: Optional[int] = None,
                ldb: Optional[int] = None, ldc: Optional[int] = None, stream=None, workspace=None) -> None:
-        """Enqueues the GEMM.  ``workspace`` (a ``DeviceArray``; stream-K plans only) replaces the
-        workspace that the library keeps per stream."""
+        """Enqueues the GEMM.  ``workspace`` (stream-K plans only) replaces the workspace that the
+        library keeps per stream: a ``DeviceArray``, or ``"static"`` for the library's fixed scratch
+        array (``rl_gemm_plan_launch_static``: no allocation on any path, a limited size)."""
         ptr = _address
         width_b = K if self.cfg.trans_b else N
         dims = (M, N, K, K if lda is None else lda, width_b if ldb is None else ldb, N if ldc is None else ldc)
-        if workspace is None:
+        if workspace == "static":
+            check(lib().rl_gemm_plan_launch_static(self.handle, ptr(A), ptr(B), ptr(Cm), *dims, _stream_handle(stream)))
+        elif workspace is None:
             check(lib().rl_gemm_plan_launch(self.handle, ptr(A), ptr(B), ptr(Cm), *dims, _stream_handle(stream)))
         else:
             check(lib().rl_gemm_plan_launch_ws(self.handle, ptr(A), ptr(B), ptr(Cm), *dims, ptr(workspace),
