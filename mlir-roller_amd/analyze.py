@@ -152,6 +152,7 @@ class TileDict:
         self.threads = 0
         self.lds_row_pad = 0
         self.pipeline_depth = DEFAULT_PIPELINE_DEPTH
+        self.stream_k = 0      # workgroups per core of a stream-K kernel; 0 = one workgroup per tile
         # analysis
         self.traffic = -1
         self.smem_cost = -1
@@ -173,6 +174,8 @@ class TileDict:
         )
         if self.wave_tile:
             text += f", wave_tile={self.wave_tile}, mfma={self.mfma}, threads={self.threads}"
+        if self.stream_k:
+            text += f", stream_k={self.stream_k}"
         return text + ")"
 
     def clone(self) -> "TileDict":
@@ -345,7 +348,25 @@ class Policy:
             return self.estimate_seconds(td)
         return (td.traffic + 1) * td.num_wave
 
-    def estimate_seconds(self, td: TileDict) -> float:
+    def simd_balance(self, block_tile: Sequence[int]) -> float:
+        """Best share of a core's matrix pipes that a workgroup computing ``block_tile`` can keep
+        busy: the tile splits into r x c wavefronts with r and c dividing its grid of (smallest)
+        matrix-instruction blocks, and a wave count that is not a multiple of the SIMD count leaves
+        pipes idle while the fullest SIMD finishes (48 x 16 is three blocks: three waves, one of
+        four SIMDs idle)."""
+        granule, simds = self._granule, self.arch.sm_partition
+        if not granule:
+            return 1.0
+        rows, cols = block_tile[0] // granule, block_tile[1] // granule
+        best = 0.0
+        for r in get_all_factors(max(rows, 1)):
+            for c in get_all_factors(max(cols, 1)):
+                waves = r * c
+                if waves * self.arch.warp_size <= 1024:
+                    best = max(best, waves / (-(-waves // simds) * simds))
+        return best or 1.0
+
+    def estimate_seconds(self, td: TileDict, stream_k: Optional[int] = None) -> float:
         """Roofline estimate of the whole GEMM with block tile ``td`` on a device with matrix
         cores.  The busiest CU works through ceil(grid / CUs) tiles.  A tile costs the larger of
         its MFMA time at the CU's share of the matrix peak and its traffic at the CU's share of
@@ -354,20 +375,41 @@ class Policy:
         fitted to a committed sweep (``calibrate.py``).  A fixed cost per tile covers filling the
         pipeline and draining the accumulators; workgroups that are resident on a CU together
         (``block_per_SM``) hide it behind one another's MFMAs, so it is paid once per group of
-        resident tiles."""
+        resident tiles.
+
+        ``stream_k`` (default: the tile's own setting) estimates the stream-K kernel instead: every
+        CU works grid / CUs tiles' worth of reduce steps, a fraction and not a whole number of
+        rounds, at a slightly lower efficiency and with a fixed cost for the pieces of split tiles."""
         a, cfg = self.arch, self.matmul_config
         m, n = td.block_tile
+        stream_k = td.stream_k if stream_k is None else stream_k
         cu_flops = a.peak_matrix_tflops * 1e12 / a.compute_max_core
         cu_bw = a.bandwidth[0] * 1e9 / a.compute_max_core
         k_steps = -(-cfg.K // td.rstep)  # the kernel runs whole K steps also where K is ragged
         tiles_per_cu = -(-td.grid_size // a.compute_max_core)
-        resident = max(1, min(td.block_per_SM, tiles_per_cu))
+        resident = max(1, min(td.block_per_SM, stream_k if stream_k else tiles_per_cu))
         base, slope = a.mfma_efficiency
-        efficiency = max(base - slope * (1.0 / m + 1.0 / n) + (a.co_resident_gain if resident > 1 else 0.0), 0.05)
+        efficiency = base - slope * (1.0 / m + 1.0 / n) + (a.co_resident_gain if resident > 1 else 0.0)
+        efficiency = max((efficiency - (a.stream_k_loss if stream_k else 0.0)) * self.simd_balance(td.block_tile), 0.05)
         t_mfma = 2.0 * m * n * k_steps * td.rstep / (cu_flops * efficiency)
         t_mem = td.traffic / cu_bw
         t_fixed = a.tile_fixed_seconds + m * n * cfg.el_bytes / cu_bw
+        if stream_k:
+            share = td.grid_size / a.compute_max_core          # tiles' worth of reduce steps per CU
+            return share * max(t_mfma, t_mem) + (-(-math.ceil(share) // resident) + 1) * t_fixed + a.stream_k_fixed_seconds
         return tiles_per_cu * max(t_mfma, t_mem) + (-(-tiles_per_cu // resident)) * t_fixed
+
+    def _choose_stream_k(self, td: TileDict) -> None:
+        """Sets ``td.stream_k`` where the estimate says that working equal shares of reduce steps
+        beats whole tiles by more than the device model's margin (the kernels exist at pipeline
+        depths with two workgroup-memory buffers and a register stage, i.e. from depth 2 on)."""
+        a = self.arch
+        td.stream_k = 0
+        if not a.stream_k_workgroups or self.pipeline_depth < 2 or self.pipeline_depth > 3:
+            return
+        workgroups = max(1, min(a.stream_k_workgroups, td.block_per_SM))
+        if self.estimate_seconds(td, workgroups) < self.estimate_seconds(td, 0) * (1.0 - a.stream_k_margin):
+            td.stream_k = workgroups
 
     def get_block_tiles_candidates(self, init_tile: List[int], rstep: int) -> List[TileDict]:
         """All valid block tiles, best first (stable with respect to enumeration order:
@@ -386,6 +428,8 @@ class Policy:
         for m, n in itertools.product(*steps):
             td = TileDict.from_block_tile([m, n], rstep, self.matmul_config, self.arch, self.pipeline_depth)
             if td.valid:
+                if granule:
+                    self._choose_stream_k(td)
                 tiles.append(td)
         return sorted(tiles, key=self._priority)
 
@@ -531,15 +575,31 @@ class Policy:
 
     # ---- top level ------------------------------------------------------------------------------
 
+    # a block tile whose plain and stream-K estimates are this close is emitted in both forms
+    STREAM_K_TOSS_UP = 0.01
+
     def emit_config(self, topk: int = 10) -> List[TileDict]:
+        """The first ``topk`` hints.  The reference completes every block tile with its first two
+        block sizes (analyze.py:367-381).  With matrix cores the second block size of a tile is a
+        near twin of the first (the fitted model: a second wave per SIMD changes nothing), so a
+        tile yields one hint and the places go to more block tiles -- and to the other form of
+        the kernel, whole tiles or stream-K, where the estimate cannot tell the two apart."""
         rstep = self._assign_reduce_step()
         hints: List[TileDict] = []
+        mfma = self.arch.has_matrix_cores
         for td in self.get_block_tiles_candidates([1, 1], rstep):
             self._expand_reduce_axis(td)
-            for hint in self.assign_thread_tile(td, 2):
+            for hint in self.assign_thread_tile(td, 1 if mfma else 2):
                 hints.append(hint)
+                if mfma and self.arch.stream_k_workgroups and 2 <= self.pipeline_depth <= 3:
+                    other = max(1, min(self.arch.stream_k_workgroups, hint.block_per_SM)) if not hint.stream_k else 0
+                    mine, its = self.estimate_seconds(hint), self.estimate_seconds(hint, other)
+                    if its < mine * (1.0 + self.STREAM_K_TOSS_UP) and len(hints) < topk:
+                        twin = hint.clone()
+                        twin.stream_k = other
+                        hints.append(twin)
                 if len(hints) >= topk:
-                    return hints
+                    return hints[:topk]
         return hints
 
 

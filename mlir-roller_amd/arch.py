@@ -64,6 +64,15 @@ class TileDevice:
     # contiguous rows, fewer loop trips: the reference's rule) or stays at the shortest step that
     # suits the loads (smaller stages, more blocks resident on a core)
     grow_reduce_step: bool = True
+    # Stream-K: workgroups per core that a kernel may keep working through equal shares of all
+    # (tile, reduce step) units instead of taking one tile each (0 = the device's kernels cannot).
+    # Such a kernel pays no round of blocks that is only partly filled; it runs its reduce steps
+    # ``stream_k_loss`` less efficiently, pays ``stream_k_fixed_seconds`` once for storing and adding up
+    # the pieces of split tiles, and is preferred when the estimate gains more than ``stream_k_margin``.
+    stream_k_workgroups: int = 0
+    stream_k_loss: float = 0.0
+    stream_k_fixed_seconds: float = 0.0
+    stream_k_margin: float = 0.0
 
     def get_avaliable_tensorintrin_shapes(self) -> List[Tuple[int, int, int]]:
         """Matrix-instruction shapes of the device (name kept from the reference, arch.py:36)."""
@@ -136,10 +145,10 @@ class MI355X(TileDevice):
     peak_matrix_tflops: float = 157.3
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
-    # (a test refits both): 0.981 for 256x256 tiles, 0.974 + 0.008 for 128x128 with two on a CU,
-    # 0.945 for 32x64
-    mfma_efficiency: Tuple[float, float] = (0.988, 0.92)
-    co_resident_gain: float = 0.008
+    # (a test refits both): 0.978 for 256x256 tiles, 0.971 + 0.011 for 128x128 with two on a CU,
+    # 0.944 for 32x64
+    mfma_efficiency: Tuple[float, float] = (0.985, 0.87)
+    co_resident_gain: float = 0.011
     tile_fixed_seconds: float = 1.0e-6
     # 16x16x4 wins on every wave tile it fits (up to 64x128; a wave keeps at most 32 blocks), by
     # 0.5-2 % in the committed sweep
@@ -148,6 +157,12 @@ class MI355X(TileDevice):
     # second workgroup on the CU would use and lengthens the fill of the pipeline (measured: 128x128
     # tiles at K steps of 32 against 64, 64x64 at 32 / 64 / 128: the shortest wins or ties)
     grow_reduce_step: bool = False
+    # fitted like the constants above (stream-K against plain kernels of the same tile on problems that
+    # fill whole rounds: 0.9 % slower); about 5 us for the pieces of a launch
+    stream_k_workgroups: int = 2
+    stream_k_loss: float = 0.009
+    stream_k_fixed_seconds: float = 5.0e-6
+    stream_k_margin: float = 0.02
     smem_cap: int = field(init=False)
     max_smem_usage: int = field(init=False)
 

@@ -37,13 +37,16 @@ from .arch import MI355X, TileDevice
 DATA_DIR = Path(__file__).resolve().parent / "calibration"
 DEFAULT_DATA = DATA_DIR / "mi355x_f32.json"
 
-# the fourteen benchmark shapes, the ragged named configuration and three mid-size cubes
+# the fourteen benchmark shapes, the ragged named configuration and three mid-size cubes ...
 SHAPES: Dict[str, Tuple[int, int, int]] = {f"M{i}": s for i, s in enumerate([
     (2048, 2048, 2048), (2048, 2048, 8192), (2048, 4096, 2048), (2048, 4096, 4096), (2048, 8192, 2048),
     (2048, 8192, 4096), (2048, 8192, 8192), (4096, 2048, 2048), (4096, 4096, 8192), (4096, 8192, 2048),
     (4096, 8192, 4096), (8192, 2048, 8192), (8192, 4096, 2048), (8192, 4096, 4096)])}
 SHAPES.update({"cfg4": (3000, 5000, 1536), "1024x1024x1024": (1024, 1024, 1024),
                "1536x1536x1536": (1536, 1536, 1536), "1000x1000x1000": (1000, 1000, 1000)})
+# ... small cubes, a tall and skinny problem, and two whose tile grids fill a fraction of their last round
+SHAPES.update({name: tuple(int(v) for v in name.split("x")) for name in (
+    "256x256x256", "512x512x512", "768x768x768", "65536x128x128", "2560x2560x2560", "1920x2880x2048")})
 
 
 MIN_FIT_MS = 0.1   # shortest measurement the efficiency fit uses
@@ -94,11 +97,16 @@ def observed_efficiency(rec: dict, arch: TileDevice) -> Optional[float]:
     return ideal_tile_seconds(m, n, K, rec["rstep"], arch) / busy
 
 
+def plain(records: Iterable[dict]) -> List[dict]:
+    """The records of kernels that take one tile per workgroup (the tile-level fits are about those)."""
+    return [r for r in records if not r.get("stream_k")]
+
+
 def best_per_block_tile(records: Iterable[dict]) -> List[dict]:
     """The fastest record of every (shape, block tile): wave split, instruction and K step are
     second-order choices that the fit of the tile-level efficiency must not see."""
     best: Dict[tuple, dict] = {}
-    for r in records:
+    for r in plain(records):
         key = (tuple(r["shape"]), tuple(r["block_tile"]))
         if key not in best or r["ms"] < best[key]["ms"]:
             best[key] = r
@@ -171,7 +179,7 @@ def fit_waves_per_simd(records: Sequence[dict], arch: Optional[TileDevice] = Non
     arch = arch or MI355X()
     one, two = arch.warp_size * arch.sm_partition, 2 * arch.warp_size * arch.sm_partition
     best: Dict[tuple, Dict[int, float]] = {}
-    for r in records:
+    for r in plain(records):
         if math.prod(r["block_tile"]) < min_tile or r["threads"] not in (one, two):
             continue
         slot = best.setdefault((tuple(r["shape"]), tuple(r["block_tile"])), {})
@@ -189,7 +197,7 @@ def fit_long_k_mfma(records: Sequence[dict], arch: Optional[TileDevice] = None) 
     (shape, block tile, wave tile) triples measured with both; the largest size whose mean is
     above 1, with every smaller size above 1 as well (``long_k_mfma_up_to``)."""
     by: Dict[tuple, Dict[int, float]] = {}
-    for r in records:
+    for r in plain(records):
         key = (tuple(r["shape"]), tuple(r["block_tile"]), tuple(r["wave_tile"]))
         slot = by.setdefault(key, {})
         slot[r["mfma"]] = min(slot.get(r["mfma"], float("inf")), r["ms"])
@@ -207,16 +215,44 @@ def fit_long_k_mfma(records: Sequence[dict], arch: Optional[TileDevice] = None) 
             "pairs": sum(len(v) for v in per_size.values())}
 
 
+def fit_stream_k(records: Sequence[dict], arch: Optional[TileDevice] = None, min_ms: float = 0.25) -> dict:
+    """What the stream-K form of a kernel costs where it has nothing to gain: over every kernel
+    measured in both forms on a problem whose tile grid fills whole rounds of CUs and that runs for
+    at least ``min_ms``, the geometric mean of time(stream-K) / time(plain), minus one
+    (``stream_k_loss``).  Per shape, the best plain time over the best stream-K time is listed for the
+    record (above 1: a stream-K kernel is the fastest one measured)."""
+    arch = arch or MI355X()
+    by: Dict[tuple, Dict[int, float]] = {}
+    for r in records:
+        key = (tuple(r["shape"]), tuple(r["block_tile"]), tuple(r["wave_tile"]), r["mfma"], r["rstep"])
+        form = 1 if r.get("stream_k") else 0
+        slot = by.setdefault(key, {})
+        slot[form] = min(slot.get(form, float("inf")), r["ms"])
+    whole = []
+    best: Dict[tuple, Dict[int, float]] = {}
+    for (shape, tile, _, _, _), t in sorted(by.items()):
+        for form, ms in t.items():
+            slot = best.setdefault(shape, {})
+            slot[form] = min(slot.get(form, float("inf")), ms)
+        tiles = (-(-shape[0] // tile[0])) * (-(-shape[1] // tile[1]))
+        if 0 in t and 1 in t and tiles % arch.compute_max_core == 0 and t[0] >= min_ms:
+            whole.append(t[1] / t[0])
+    if not whole:
+        raise ValueError("no kernel was measured in both forms on a problem that fills whole rounds")
+    gains = {"x".join(str(v) for v in shape): round(t[0] / t[1], 4) for shape, t in sorted(best.items()) if 0 in t and 1 in t}
+    return {"stream_k_loss": round(_geo_mean(whole) - 1.0, 3), "pairs": len(whole), "best_plain_over_best_stream_k": gains}
+
+
 # ---------------------------------------------------------------------------------------------
 # replaying the policy on a data set
 # ---------------------------------------------------------------------------------------------
 
 def _key_of_hint(hint: TileDict) -> tuple:
-    return (tuple(hint.block_tile), tuple(hint.wave_tile), hint.mfma, hint.rstep)
+    return (tuple(hint.block_tile), tuple(hint.wave_tile), hint.mfma, hint.rstep, 1 if hint.stream_k else 0)
 
 
 def _key_of_record(rec: dict) -> tuple:
-    return (tuple(rec["block_tile"]), tuple(rec["wave_tile"]), rec["mfma"], rec["rstep"])
+    return (tuple(rec["block_tile"]), tuple(rec["wave_tile"]), rec["mfma"], rec["rstep"], 1 if rec.get("stream_k") else 0)
 
 
 def check(records: Sequence[dict], arch: Optional[TileDevice] = None, topk: int = 4, depth: int = DEFAULT_PIPELINE_DEPTH) -> List[dict]:
@@ -265,7 +301,12 @@ def candidate_hints(cfg: MatmulConfig, arch: TileDevice, topk: int, depth: int =
             done = policy._assign_wave_tiles(td, block_size)
             if not done:
                 continue
-            out.extend(done)
+            for hint in done:
+                # both forms of every kernel, whole tiles and stream-K, whatever the estimate prefers
+                for form in ((0, max(1, min(arch.stream_k_workgroups, hint.block_per_SM))) if arch.stream_k_workgroups and 2 <= depth <= 3 else (0,)):
+                    twin = hint.clone()
+                    twin.stream_k = form
+                    out.append(twin)
             sizes += 1
             if sizes == 2:
                 break
@@ -308,7 +349,7 @@ def measure(shape_names: Sequence[str], topk: int, depth: int = DEFAULT_PIPELINE
             for (rank, hint, g, _), ms in zip(part, times):
                 records.append({"shape": list(shape), "block_tile": list(hint.block_tile), "wave_tile": list(hint.wave_tile),
                                 "mfma": hint.mfma, "rstep": hint.rstep, "threads": hint.threads, "edge": g.edge,
-                                "direct": g.direct, "rank_when_measured": rank, "ms": round(ms, 6)})
+                                "direct": g.direct, "stream_k": g.streamk, "rank_when_measured": rank, "ms": round(ms, 6)})
         best = min((r for r in records if r["shape"] == list(shape)), key=lambda r: r["ms"])
         say(f"[calibrate] {name} {shape}: {len(cands)} kernels, best {best['ms']:.4f} ms "
             f"({2.0 * M * N * K / best['ms'] / 1e9:.1f} TFLOP/s) rank {best['rank_when_measured']} {best['block_tile']}/{best['wave_tile']}/mi{best['mfma']}/k{best['rstep']}")
@@ -329,8 +370,11 @@ def main(argv=None) -> int:
     sub = ap.add_subparsers(dest="cmd", required=True)
     m = sub.add_parser("measure")
     m.add_argument("--out", default=str(DEFAULT_DATA))
-    m.add_argument("--topk", type=int, default=48)
+    m.add_argument("--topk", type=int, default=96, help="kernels per shape, both forms (whole tiles and stream-K) counted")
     m.add_argument("--shapes", nargs="*", default=list(SHAPES))
+    pc = sub.add_parser("precompile", help="no GPU: fill the code-object cache with the kernels that `measure` will time")
+    pc.add_argument("--topk", type=int, default=96)
+    pc.add_argument("--shapes", nargs="*", default=list(SHAPES))
     f = sub.add_parser("fit")
     f.add_argument("--data", default=str(DEFAULT_DATA))
     c = sub.add_parser("check")
@@ -338,6 +382,22 @@ def main(argv=None) -> int:
     c.add_argument("--topk", type=int, default=4)
     args = ap.parse_args(argv)
 
+    if args.cmd == "precompile":
+        from . import hip
+        from .roller import hint_to_gemm_config
+        todo = []
+        for name in args.shapes:
+            cfg = MatmulConfig(*shape_of(name), 32)
+            for hint in candidate_hints(cfg, MI355X(), args.topk):
+                try:
+                    g = hint_to_gemm_config(cfg, hint, DEFAULT_PIPELINE_DEPTH)
+                    hip.config_check(g)
+                    todo.append(g)
+                except Exception:
+                    pass
+        failed = hip.precompile_many(todo)
+        print(f"{len(set(todo))} kernels, {len(failed)} failed to compile")
+        return 1 if failed else 0
     if args.cmd == "measure":
         data = measure(args.shapes, args.topk)
         out = Path(args.out)
@@ -354,6 +414,12 @@ def main(argv=None) -> int:
         waves = fit_waves_per_simd(data["records"])
         print(f"fitted waves_per_partition = {waves['waves_per_partition']} (two waves per SIMD take {waves['two_over_one']:.4f} x "
               f"the time of one, {waves['pairs']} block tiles); arch.MI355X has {now.waves_per_partition}")
+        try:
+            sk = fit_stream_k(data["records"])
+            print(f"fitted stream_k_loss = {sk['stream_k_loss']} ({sk['pairs']} kernels in both forms on whole rounds); arch.MI355X has "
+                  f"{now.stream_k_loss}; best plain over best stream-K per shape: {sk['best_plain_over_best_stream_k']}")
+        except ValueError as e:
+            print(f"stream_k_loss not fitted: {e}")
         instr = fit_long_k_mfma(data["records"])
         print(f"fitted long_k_mfma_up_to = {instr['long_k_mfma_up_to']} (32x32x2 over 16x16x4 by wave-tile elements: "
               f"{instr['mi32_over_mi16_by_wave_tile_elems']}); arch.MI355X has {now.long_k_mfma_up_to}")

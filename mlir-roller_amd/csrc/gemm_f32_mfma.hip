@@ -899,7 +899,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     {
       const __amdgpu_buffer_rsrc_t wr = make_rsrc(sk_slots + (long)my_slot * (BM * BN), (long)BM * BN * 4);
 #pragma unroll
-      for (int bi = 0; bi < TM; ++bi)
+      for (int bi = 0; bi < TM; ++bi) {
 #pragma unroll
         for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
@@ -907,6 +907,8 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
             const v4f v = {acc[bi][bj][4 * c], acc[bi][bj][4 * c + 1], acc[bi][bj][4 * c + 2], acc[bi][bj][4 * c + 3]};
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), wr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, SK_COHERENT);
           }
+        __builtin_amdgcn_sched_barrier(0);   // (a row of blocks at a time, see the reading side)
+      }
     }
     // the piece has arrived in memory; then count this workgroup in
     WAIT_VMCNT(0);
@@ -920,7 +922,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
       auto add_piece = [&](auto is_first, unsigned slot) __attribute__((always_inline)) {
         const __amdgpu_buffer_rsrc_t rr = make_rsrc(sk_slots + (long)slot * (BM * BN), (long)BM * BN * 4);
 #pragma unroll
-        for (int bi = 0; bi < TM; ++bi)
+        for (int bi = 0; bi < TM; ++bi) {
 #pragma unroll
           for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
@@ -929,6 +931,10 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #pragma unroll
               for (int e = 0; e < 4; ++e) acc[bi][bj][4 * c + e] = decltype(is_first)::value ? v[e] : acc[bi][bj][4 * c + e] + v[e];
             }
+          // one row of blocks at a time: left alone, the scheduler issues every load of the piece first and
+          // the kernel needs a second set of accumulator registers for them (one wave per SIMD instead of two)
+          __builtin_amdgcn_sched_barrier(0);
+        }
       };
       add_piece(int_c<1>{}, 2 * first_wg + 1);
       for (unsigned piece = 1; piece < pieces; ++piece) add_piece(int_c<0>{}, 2 * (first_wg + piece));

@@ -96,6 +96,8 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
         # 0: every extent is a whole number of tiles; 2: only M or N is ragged; 1: K is ragged too
         edge=(0 if (M % bm == 0 and N % bn == 0) else 2) if K % bk == 0 else 1,
         swz=3, group=8, accum=1 if accumulate else 0, direct=direct, trans_b=1 if trans_b else 0,
+        # the stream-K form of the kernel exists on the pipelined loop only
+        streamk=int(getattr(hint, "stream_k", 0)) if stages == 3 else 0,
     )
 
 

@@ -19,7 +19,8 @@ from __future__ import annotations
 from typing import List, Optional, Sequence, Tuple
 
 DEFAULT_TOPK = 4      # hints tried per shape (the reference: 20, benchmark.py:10)
-TIE_MARGIN = 0.005    # relative spread of two timings of the same kernel a few milliseconds apart
+TIE_MARGIN = 0.01     # relative spread of two timings of the same kernel: about half a percent a few milliseconds
+                      # apart, up to three percent for small-tile kernels between one batch of launches and the next
 RAMP_MS = 40.0        # continuous load queued ahead of a timed region: the engine clock drops within
                       # microseconds of the GPU going idle and needs about 25 ms to come back
 
