@@ -217,6 +217,8 @@ def main() -> int:
     ap.add_argument("--topk", type=int, default=DEFAULT_TOPK)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--retune", action="store_true", help="ignore remembered winners")
+    ap.add_argument("--depth", type=int, default=None, help="pipeline depth 1..5 (default: the sweep's, 3; the reference's 2 is the same kernel)")
+    ap.add_argument("--trans-b", action="store_true", help="the kernels that take the second operand as Bt[N, K]")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--lean", action="store_true",
                     help="profiling mode: no cold-compile timing, no named configurations, no clock probe")
@@ -233,8 +235,10 @@ def main() -> int:
     from mlir_roller_amd import hip, tuner
     from mlir_roller_amd.analyze import MatmulConfig, get_roller_hints
     from mlir_roller_amd.arch import MI355X
-    from mlir_roller_amd.benchmark import PIPELINE_DEPTH, README_SHAPES
+    from mlir_roller_amd.benchmark import README_SHAPES
+    from mlir_roller_amd import benchmark as sweep
     from mlir_roller_amd.hip import DeviceArray, Event, GemmConfig, GemmPlan, Module, Stream
+    PIPELINE_DEPTH = sweep.PIPELINE_DEPTH if args.depth is None else args.depth
     from mlir_roller_amd.roller import gemm_errors, hint_to_gemm_config, make_inputs
 
     if args.workload == "sweep":
@@ -266,7 +270,7 @@ def main() -> int:
     cache_dir = Path(os.environ.get("ROLLER_HIP_CACHE", str(hip.DEFAULT_CACHE_DIR)))
     cache_dir.mkdir(parents=True, exist_ok=True)
     template_id = hashlib.sha1(hip.template_source().encode()).hexdigest()[:12]
-    tuned_path = cache_dir / f"tuned_{template_id}_top{args.topk}_d{PIPELINE_DEPTH}.json"
+    tuned_path = cache_dir / f"tuned_{template_id}_top{args.topk}_d{PIPELINE_DEPTH}{'_tb' if args.trans_b else ''}.json"
     tuned = {}
     if tuned_path.exists() and not args.retune:
         try:
@@ -302,7 +306,7 @@ def main() -> int:
         M, N, K = shape
         cfg = MatmulConfig(M, N, K, 32)
         A, B = make_inputs(cfg, args.seed, distribution)
-        bufs = (DeviceArray.from_host(A), DeviceArray.from_host(B), DeviceArray.zeros((M, N)))
+        bufs = (DeviceArray.from_host(A), DeviceArray.from_host(B.T if args.trans_b else B), DeviceArray.zeros((M, N)))
 
         t0 = time.perf_counter()
         hints = get_roller_hints(cfg, arch, topk=args.topk, pipeline_depth=PIPELINE_DEPTH)
@@ -311,7 +315,7 @@ def main() -> int:
         usable = []  # (rank, GemmConfig, hint text)
         for rank, hint in enumerate(hints, 1):
             try:
-                g = hint_to_gemm_config(cfg, hint, PIPELINE_DEPTH)
+                g = hint_to_gemm_config(cfg, hint, PIPELINE_DEPTH, trans_b=args.trans_b)
                 hip.config_check(g)
                 usable.append((rank, g, repr(hint)))
                 candidates_seen[g] = None
@@ -322,9 +326,14 @@ def main() -> int:
         key = f"{M}x{N}x{K}:{distribution}"
         order = []   # ranks in the order in which verification tries them
         timings = []
-        if key in tuned and any(r == tuned[key]["rank"] for r, _, _ in usable):
-            order = [tuned[key]["rank"]]
-            timings = [tuple(t) for t in tuned[key].get("timings", [])]
+        # A remembered winner is a kernel (its tag), not a rank: ranks move when the policy's constants
+        # do.  It is reused only if today's hints still hold that kernel, at whatever rank.
+        remembered = [r for r, g, _ in usable if key in tuned and g.tag() == tuned[key].get("kernel")]
+        replayed = bool(remembered)
+        if replayed:
+            order = [remembered[0]]
+            by_tag = {g.tag(): r for r, g, _ in usable}
+            timings = [(by_tag[tag], ms) for tag, ms in tuned[key].get("timings", []) if tag in by_tag]
             from_cache_shapes += 1
         else:
             t0 = time.perf_counter()
@@ -377,11 +386,14 @@ def main() -> int:
         if chosen is None:
             raise RuntimeError(f"{name}: every hint failed verification")
         rank, g, text, plan, rep = chosen
-        tuned[key] = {"rank": rank, "timings": [list(t) for t in timings]}
+        tag_of = {r: gg.tag() for r, gg, _ in usable}
+        tuned[key] = {"kernel": g.tag(), "timings": [[tag_of[r], t] for r, t in timings if r in tag_of]}
         summary = tuner.summarise(timings, rank)
+        summary["tuning"] = "from_cache" if replayed else "this_run"
         ms = dict(timings).get(rank, float("nan"))
         log(f"[bench] {name} {shape}: rank {rank}/{len(hints)} {g.tag()}  {ms:.4f} ms  "
-            f"{2.0 * M * N * K / ms / 1e9:.1f} TFLOP/s  normwise {rep['normwise']:.2e} max_abs {rep['max_abs']:.2e}  {summary}")
+            f"{2.0 * M * N * K / ms / 1e9:.1f} TFLOP/s " + ("(tuning figures replayed from an earlier run's memory) " if replayed else "")
+            + f" normwise {rep['normwise']:.2e} max_abs {rep['max_abs']:.2e}  {summary}")
         return {"name": name, "shape": shape, "plan": plan, "bufs": bufs, "rank": rank, "hints": len(hints), "tuned_ms": ms,
                 "summary": summary, "cfg": g, "hint": text, "rep": rep, "host_ms": t_host * 1e3, "dist": distribution}
 
@@ -545,7 +557,7 @@ def main() -> int:
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": workload, "launches_per_step": launches, "inputs": f"{dist}, seed {args.seed}",
-                   "topk": args.topk, "tie_margin": TIE_MARGIN, "pipeline_depth": PIPELINE_DEPTH},
+                   "topk": args.topk, "tie_margin": TIE_MARGIN, "pipeline_depth": PIPELINE_DEPTH, "trans_b": bool(args.trans_b)},
         "pct_of_fp32_matrix_peak": round(100 * tflops / PEAK_TFLOPS, 2),
         "roofline": {
             "bound": "mfma", "achieved": round(tflops, 3), "peak": PEAK_TFLOPS, "unit": "TFLOP/s",

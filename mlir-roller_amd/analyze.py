@@ -99,15 +99,26 @@ def compute_memory_traffic(output_tile: List[int], matmul_config: MatmulConfig, 
 DEFAULT_PIPELINE_DEPTH = 3
 
 
+def kernel_stages(pipeline_depth: int) -> int:
+    """STAGES of the kernel template for a ``pipeline_depth`` as the reference means it, the number
+    of workgroup-memory buffers per operand (/root/reference/src/roller.py:200-205, :385): 1 -> one
+    buffer, nothing overlapped; 2 -> two buffers and the fully pipelined loop (template STAGES 3: the
+    template's own STAGES 2, two buffers with the loads staged through registers and waited for in
+    the open, is kept for explicit configurations only -- it is 13 % slower and needs the same LDS);
+    3 -> the same kernel (the depth the MI355X sweep asks for); 4, 5 -> three and four buffers."""
+    depth = max(1, int(pipeline_depth))
+    return 3 if depth == 2 else depth
+
+
 def loads_go_direct_to_lds(matmul_config: "MatmulConfig", block_tile: Sequence[int], rstep: int,
                            pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> bool:
     """Whether the MFMA kernel built for this tile uses its direct-to-LDS path (unpadded,
-    XOR-swizzled rows; no staging registers): only at pipeline depth 3, with 128-bit global
-    accesses (K and N multiples of 4), a power-of-two reduce step, and operand tiles that are
-    whole waves of 16-byte units.  The policy's LDS and register models and the mapping from a
-    hint to template parameters all ask this one function."""
+    XOR-swizzled rows; no staging registers): on the pipelined loop (pipeline depth 2 and up), with
+    128-bit global accesses (K and N multiples of 4), a power-of-two reduce step, and operand tiles
+    that are whole waves of 16-byte units.  The policy's LDS and register models and the mapping
+    from a hint to template parameters all ask this one function."""
     m, n = block_tile
-    return (pipeline_depth >= 3 and matmul_config.K % 4 == 0 and matmul_config.N % 4 == 0
+    return (kernel_stages(pipeline_depth) >= 3 and matmul_config.K % 4 == 0 and matmul_config.N % 4 == 0
             and rstep & (rstep - 1) == 0 and (m * rstep // 4) % 64 == 0 and (rstep * n // 4) % 64 == 0)
 
 

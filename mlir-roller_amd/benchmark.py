@@ -50,7 +50,10 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = DEFAULT_T
               csv_path: Optional[os.PathLike] = "benchmark_results.csv",
               dump_path: Optional[os.PathLike] = None, repeat_times: int = 20,
               distribution: str = "uniform", seed: int = 0, counters: bool = False,
-              vendor: bool = False) -> pd.DataFrame:
+              vendor: bool = False, pipeline_depth: Optional[int] = None, trans_b: bool = False) -> pd.DataFrame:
+    """The reference's sweep (benchmark.py:10-95) with its table.  ``pipeline_depth`` (default: the
+    sweep's, 3; the reference's own 2 is the same kernel) and ``trans_b`` (second operand given as
+    Bt[N, K]) select the kernel variant that is timed."""
     arch = arch or MI355X()
     peak_tflops = arch.peak_matrix_tflops or float("nan")
     results = []
@@ -84,7 +87,7 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = DEFAULT_T
 
         # 2. roller hints
         # the reference runs depth 2 (benchmark.py:29); here 3 = two LDS buffers + a register stage
-        pipeline_depth = PIPELINE_DEPTH
+        pipeline_depth = PIPELINE_DEPTH if pipeline_depth is None else int(pipeline_depth)
         print(f"Generating and testing {topk} roller hints...")
         t0 = time.perf_counter()
         try:
@@ -99,8 +102,8 @@ def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = DEFAULT_T
         for i, hint in enumerate(hints):
             print(f"  Testing hint {i + 1}/{len(hints)}: {hint}")
             try:
-                func = Compiler(config, hint, pipeline_depth,
-                                dump_path=Path(dump_path) if dump_path else None).compile()
+                func = Compiler(config, hint, pipeline_depth, dump_path=Path(dump_path) if dump_path else None,
+                                **({"trans_b": True} if trans_b else {})).compile()
                 compile_s += func.compile_ms / 1e3
                 t, gflops = run_eval(func, pipeline_depth, hint, repeat_times=repeat_times,
                                      seed=seed, distribution=distribution)
@@ -228,6 +231,8 @@ def main(argv=None) -> None:
     ap.add_argument("--dump", default=None, help="directory for kernel source / ISA dumps")
     ap.add_argument("--plot", default=None, help="write a bar chart of the sweep to this image file")
     ap.add_argument("--vendor", action="store_true", help="also time rocBLAS sgemm on the GPU (the reference's cuBLAS column)")
+    ap.add_argument("--depth", type=int, default=None, help="pipeline depth 1..5 (default 3; the reference's 2 is the same kernel)")
+    ap.add_argument("--trans-b", action="store_true", help="time the kernels that take the second operand as Bt[N, K]")
     ap.add_argument("--counters", action="store_true",
                     help="add rocprofv3 counter columns (MFMA busy %%, LDS bank conflicts, HBM-side GB/s); several extra runs per shape")
     args = ap.parse_args(argv)
@@ -246,7 +251,7 @@ def main(argv=None) -> None:
         except ValueError:
             ap.error(f"--shapes {args.shapes}: expected readme, full, mid or a comma-separated list of MxNxK")
     df = benchmark(shapes, topk=args.topk, baseline=not args.no_baseline, csv_path=args.csv, dump_path=args.dump,
-                   counters=args.counters, vendor=args.vendor)
+                   counters=args.counters, vendor=args.vendor, pipeline_depth=args.depth, trans_b=args.trans_b)
     if args.plot:
         print(f"Chart saved to {plot_results(df, args.plot)}")
 

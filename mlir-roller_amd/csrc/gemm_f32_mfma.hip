@@ -21,12 +21,14 @@
 //   WM, WN      wave tile; (BM/WM)*(BN/WN) waves of 64 lanes form the workgroup
 //   MI          32 -> v_mfma_f32_32x32x2_f32, 16 -> v_mfma_f32_16x16x4_f32
 //   STAGES      pipeline depth: 1 = one LDS buffer, nothing overlapped; 2 = two LDS buffers, the
-//               global loads of step k+1 in flight during the MFMAs of step k; 3 = two LDS buffers
-//               plus a register stage: global loads run two steps ahead, and the LDS fragments of
-//               the next MFMA group are read while the current group executes, also across the
-//               barrier that ends a K step; 4 and 5 (DIRECT only) = the same with three and four
-//               LDS buffers, so that loads run two and three K steps ahead of the MFMAs -- for
-//               short K steps whose MFMA time does not cover a trip to HBM
+//               global loads of step k+1 staged through registers during the MFMAs of step k and
+//               written to LDS after them; 3 = two LDS buffers and the fully pipelined loop: the
+//               loads of a tile are issued a whole K step ahead (DIRECT: straight into the other
+//               LDS buffer; staged: into registers, two steps ahead of their use), the LDS
+//               fragments of the next MFMA group are read while the current group executes, also
+//               across the barrier that ends a K step; 4 and 5 (DIRECT only) = the same with
+//               three and four LDS buffers, so that loads run two and three K steps ahead of the
+//               MFMAs -- for short K steps whose MFMA time does not cover a trip to HBM
 //   PAD_A,PAD_B extra floats per LDS row of the A tile ([BM][BK+PAD_A]) and B tile ([BK][BN+PAD_B]);
 //               LDS holds the A tiles of all buffers first, then the B tiles, so that both tiles of
 //               either buffer are within the 64 KB immediate offset of an LDS read

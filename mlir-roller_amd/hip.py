@@ -249,19 +249,85 @@ def device_info() -> DeviceProps:
 
 
 def set_cache_dir(path: Optional[os.PathLike]) -> None:
+    global _cache_dir_override
     check(lib().rl_set_cache_dir(str(path).encode() if path else None))
+    _cache_dir_override = str(path) if path else None
 
 
 def synchronize() -> None:
     check(lib().rl_sync())
 
 
+_roctx = None
+
+
+def _roctx_lib():
+    """libroctx64 (ROCm's marker API), or False if it cannot be loaded."""
+    global _roctx
+    if _roctx is None:
+        _roctx = False
+        for name in ("libroctx64.so", "libroctx64.so.4", str(ROCM / "lib" / "libroctx64.so")):
+            try:
+                handle = C.CDLL(name)
+                handle.roctxRangePushA.argtypes = [C.c_char_p]
+                handle.roctxRangePushA.restype = C.c_int
+                handle.roctxRangePop.restype = C.c_int
+                _roctx = handle
+                break
+            except (OSError, AttributeError):
+                continue
+    return _roctx
+
+
+class profiler_range:
+    """``with profiler_range("name"):`` -- a roctx range that ``rocprofv3 --marker-trace`` shows, the
+    counterpart of ``cupyx.profiler.time_range`` (roller.py:556).  Does nothing when the marker
+    library is not installed."""
+
+    def __init__(self, name: str):
+        self.name = name.encode()
+        self.pushed = False
+
+    def __enter__(self):
+        lib_ = _roctx_lib()
+        if lib_:
+            lib_.roctxRangePushA(self.name)
+            self.pushed = True
+        return self
+
+    def __exit__(self, *exc):
+        if self.pushed:
+            _roctx_lib().roctxRangePop()
+        return False
+
+
 # --------------------------------------------------------------------------------------------
 # device memory, streams, events
 # --------------------------------------------------------------------------------------------
 
+class DevicePtr(int):
+    """A device address.  An ``int`` in every respect (arithmetic, formatting, ctypes pointer
+    arguments) that kernel launches recognise as an address: it is passed as an 8-byte pointer
+    whatever its value, where a plain ``int`` is a 4-byte kernel parameter."""
+
+    __slots__ = ()
+
+    def __repr__(self) -> str:
+        return f"DevicePtr({int(self):#x})"
+
+
+class _DataView:
+    """``array.data.ptr``, the spelling of CuPy that the reference's launch uses (roller.py:548)."""
+
+    __slots__ = ("ptr",)
+
+    def __init__(self, ptr: int):
+        self.ptr = DevicePtr(ptr)
+
+
 class DeviceArray:
-    """A row-major fp32 (or any dtype) array in HBM; frees its allocation when collected."""
+    """A row-major fp32 (or any dtype) array in HBM; frees its allocation when collected.
+    ``ptr`` (and ``data.ptr``, as in CuPy) is its device address as a ``DevicePtr``."""
 
     def __init__(self, shape: Sequence[int], dtype=np.float32):
         init()
@@ -270,7 +336,11 @@ class DeviceArray:
         self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
         p = C.c_void_p()
         check(lib().rl_malloc(C.byref(p), self.nbytes))
-        self.ptr = p.value or 0
+        self.ptr = DevicePtr(p.value or 0)
+
+    @property
+    def data(self) -> _DataView:
+        return _DataView(self.ptr)
 
     @classmethod
     def from_host(cls, host: np.ndarray) -> "DeviceArray":
@@ -302,7 +372,7 @@ class DeviceArray:
     def free(self) -> None:
         if getattr(self, "ptr", 0):
             lib().rl_free(self.ptr)
-            self.ptr = 0
+            self.ptr = DevicePtr(0)
 
     def __del__(self):
         try:
@@ -461,14 +531,16 @@ class Ptr:
 
 def _pack_arg(a):
     """One kernel argument as the ctypes object whose storage ``hipModuleLaunchKernel`` reads.
-    The width is decided by the argument's type, never by its value: ``DeviceArray``, ``Ptr``
-    and ``c_void_p`` are 8-byte pointers; a Python or numpy integer is a 4-byte ``int``
+    The width is decided by the argument's type, never by its value: ``DeviceArray``, ``Ptr``,
+    ``DevicePtr`` (what ``array.ptr`` and ``array.data.ptr`` are) and ``c_void_p`` are 8-byte pointers; a Python or numpy integer is a 4-byte ``int``
     (``OverflowError`` if it does not fit -- use ``ctypes.c_long`` for a 64-bit parameter and
     ``Ptr`` for an address); a float is a 4-byte ``float``; ctypes scalars pass through."""
     if isinstance(a, DeviceArray):
         return C.c_void_p(a.ptr)
     if isinstance(a, Ptr):
         return C.c_void_p(a.address)
+    if isinstance(a, DevicePtr):
+        return C.c_void_p(int(a))
     if isinstance(a, (C._SimpleCData,)):
         return a
     if isinstance(a, (bool, np.bool_)):
@@ -530,35 +602,44 @@ def _address(x) -> int:
     return int(x)
 
 
-def _precompile_worker(cfg_values: tuple) -> tuple:
+def _precompile_worker(job: tuple) -> tuple:
+    cache_dir, cfg_values = job
     cfg = GemmConfig(*cfg_values)
     try:
+        if cache_dir:
+            set_cache_dir(cache_dir)
         return cfg_values, precompile(cfg), ""
     except HipError as e:
         return cfg_values, 0, str(e)
 
 
+_cache_dir_override: Optional[str] = None
+
+
 def precompile_many(configs: Sequence[GemmConfig], jobs: Optional[int] = None) -> dict:
     """Fills the on-disk cache for ``configs`` with ``jobs`` worker processes (hiprtc is
     single-threaded and needs no GPU; default: the CPUs this process may run on, at most 16).
-    Returns ``{config: error text}`` for the ones that failed; the rest are in the cache."""
+    The workers are fresh interpreters (``spawn``): a fork of a process that has initialised the
+    GPU would inherit its runtime's threads and queues.  They get the parent's cache directory
+    explicitly.  Returns ``{config: error text}`` for the ones that failed; the rest are in the cache."""
     import concurrent.futures as cf
+    import multiprocessing as mp
 
     todo = list(dict.fromkeys(configs))
     if jobs is None:
         jobs = min(16, len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1))
-    values = [tuple(getattr(c, f.name) for f in fields(c)) for c in todo]
+    lib()
+    cache_dir = _cache_dir_override or os.environ.get("ROLLER_HIP_CACHE", str(DEFAULT_CACHE_DIR))
+    work = [(cache_dir, tuple(getattr(c, f.name) for f in fields(c))) for c in todo]
     failed = {}
     if jobs <= 1 or len(todo) <= 1:
-        results = map(_precompile_worker, values)
+        results = list(map(_precompile_worker, work))
     else:
-        pool = cf.ProcessPoolExecutor(max_workers=min(jobs, len(todo)))
-        results = pool.map(_precompile_worker, values, chunksize=1)
+        with cf.ProcessPoolExecutor(max_workers=min(jobs, len(todo)), mp_context=mp.get_context("spawn")) as pool:
+            results = list(pool.map(_precompile_worker, work, chunksize=4))
     for vals, _, err in results:
         if err:
             failed[GemmConfig(*vals)] = err
-    if jobs > 1 and len(todo) > 1:
-        pool.shutdown()
     return failed
 
 

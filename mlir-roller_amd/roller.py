@@ -22,7 +22,8 @@ from typing import Optional, Tuple
 import numpy as np
 
 from . import hip
-from .analyze import MatmulConfig, TileDict, get_roller_hints, lds_row_pad, loads_go_direct_to_lds, split_block_over_waves
+from .analyze import (MatmulConfig, TileDict, get_roller_hints, kernel_stages, lds_row_pad, loads_go_direct_to_lds,
+                      split_block_over_waves)
 from .arch import MI355X
 from .hip import DeviceArray, Event, GemmConfig, GemmPlan
 from .utils import get_block_dims
@@ -41,7 +42,8 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
 
     block_tile -> BM, BN; rstep -> BK; wave_tile -> WM, WN (derived from the thread count when
     the hint comes from a device model without matrix cores); pipeline_depth -> pipeline stages
-    (the template has 1 to 3; from 2 on it keeps two LDS buffers).  Ragged problems switch on predication, and problems whose K, N
+    (``kernel_stages``: the reference's depth 2 and the sweep's depth 3 are the same kernel, two LDS
+    buffers and the pipelined loop; 4 and 5 add buffers).  Ragged problems switch on predication, and problems whose K, N
     are not multiples of 4 fall back to dword global accesses.  ``trans_b`` selects the kernel
     whose second operand is stored as Bt[N, K].
     """
@@ -61,7 +63,7 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
                              f"for {threads} threads and reduce step {bk}")
         (wm, wn), mi = split
     M, N, K = config.M, config.N, config.K
-    stages = max(1, min(GemmConfig.MAX_STAGES, int(pipeline_depth)))
+    stages = min(GemmConfig.MAX_STAGES, kernel_stages(pipeline_depth))
     vec = 4 if (K % 4 == 0 and N % 4 == 0) else 1
     # Depths 4 and 5 (three and four LDS buffers) exist on the direct-to-LDS path only, for tiles
     # that divide evenly over the threads and fit the CU's LDS; otherwise the deepest depth that
@@ -167,9 +169,10 @@ class Compiler:
     """Same constructor and ``compile()`` as the reference's ``Compiler`` (roller.py:345-387).
 
     ``dump_path`` receives ``kernel.hip`` (template source with the chosen parameters as
-    defines), ``kernel.json`` (parameters and register/LDS usage) and, when ``hipcc`` is on the
-    PATH, ``kernel.s`` (gfx950 assembly) -- the counterparts of the reference's
-    ``transformed.mlir`` / ``llvm.mlir`` / ``kernel.ptx`` dumps.
+    defines), ``kernel.json`` (parameters and register/LDS usage), ``build.log`` (what hiprtc
+    printed for this kernel, or a line saying that the code object came from the cache) and, when
+    ``hipcc`` is on the PATH, ``kernel.s`` (gfx950 assembly) -- the counterparts of the reference's
+    ``transformed.mlir`` / ``llvm.mlir`` / ``kernel.ptx`` dumps (roller.py:369-371, :480-495, :502).
     """
 
     def __init__(self, config: MatmulConfig, hint: TileDict, pipeline_depth: int = 2,
@@ -200,6 +203,11 @@ class Compiler:
         info = {"config": vars(g), "lds_bytes": handle.shared_mem_bytes, "threads": handle.threads,
                 "resources": handle.plan.resources(), "compile_ms": handle.compile_ms}
         (out / "kernel.json").write_text(json.dumps(info, indent=1))
+        log = handle.plan.build_log()
+        if not log:
+            log = ("(no compiler output: the code object came from the in-process or on-disk cache)\n" if handle.compile_ms == 0
+                   else "(hiprtc compiled this kernel without a message)\n")
+        (out / "build.log").write_text(log)
         hipcc = shutil.which("hipcc")
         if hipcc:
             subprocess.run([hipcc, "--offload-arch=gfx950", "-O3", "--cuda-device-only", "-S",
@@ -310,7 +318,10 @@ def run_eval(cuda_func: KernelHandle, pipeline_depth, hint: TileDict, repeat_tim
         if not info["ok"]:
             raise AssertionError(f"GEMM result outside tolerance for {hint}: {info}")
 
-    cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
+    # one launch inside a named range, for a profiler to find (the reference: an NVTX range "roller",
+    # roller.py:556-562; here a roctx range of the same name when the marker library is there)
+    with hip.profiler_range("roller"):
+        cuda_func(grid_dims, block_dims, args, shared_mem=shared_memory_usage)
     # The reference warms up with 10 launches.  On MI355X the engine clock drops as soon as the
     # GPU idles (here: during the check above) and needs about 25 ms of load to come back, so
     # the warm-up is extended to cover WARMUP_MS; it runs straight into the timed launches.

@@ -553,6 +553,7 @@ def test_named_configs_full_size_through_policy_and_compiler(device, name, shape
         hip.synchronize()
         assert np.array_equal(got, dC.get())                         # bit-for-bit across runs
     assert (tmp_path / "kernel.hip").exists() and (tmp_path / "kernel.json").exists()
+    assert (tmp_path / "build.log").read_text().strip()         # the compiler's output, or a line that says there was none
 
 
 TUNER_TOPK = 8   # at least what the tuner tries by default, with room for a user's --topk 8

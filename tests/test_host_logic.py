@@ -16,10 +16,13 @@ def test_hint_to_gemm_config_aligned_problem():
     hint = next(h for h in get_roller_hints(cfg, MI355X(), 20) if h.block_tile == [256, 256])
     g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=2)
     assert (g.bm, g.bn, g.bk, g.wm, g.wn, g.mi) == (256, 256, hint.rstep, *hint.wave_tile, hint.mfma)
-    assert (g.stages, g.vec, g.edge, g.accum, g.direct) == (2, 4, 0, 0, 0)
-    assert ((g.bk + g.pad_a) // 4) % 2 == 1          # odd number of 16-byte units per LDS-A row
+    # the reference's depth (two shared-memory buffers, benchmark.py:29) is the pipelined direct-to-LDS kernel:
+    # template STAGES 3 keeps two LDS buffers too; swizzle instead of padding
+    assert (g.stages, g.vec, g.edge, g.accum, g.direct, g.pad_a, g.pad_b) == (3, 4, 0, 0, 1, 0, 0)
     g3 = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3)
-    assert (g3.stages, g3.direct, g3.pad_a, g3.pad_b) == (3, 1, 0, 0)   # direct-to-LDS: swizzle instead of padding
+    assert g3 == g                                                       # depth 3, the sweep's, is the same kernel
+    g1 = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=1)
+    assert (g1.stages, g1.direct) == (1, 0) and ((g1.bk + g1.pad_a) // 4) % 2 == 1   # staged: odd number of 16-byte units per LDS-A row
     assert g.threads == hint.threads and g.lds_bytes <= 160 * 1024
     assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=1).stages == 1
     assert roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3).stages == 3
@@ -243,6 +246,14 @@ def test_kernel_arguments_are_typed_by_type_not_by_value():
     from mlir_roller_amd import hip
     assert C.sizeof(hip._pack_arg(hip.Ptr(0))) == 8 and hip._pack_arg(hip.Ptr(0)).value is None   # NULL stays a pointer
     assert C.sizeof(hip._pack_arg(hip.Ptr(4096))) == 8
+    # what array.ptr / array.data.ptr are: an int that launches pass as an address, as the reference's call
+    # func(grid, block, (dA.data.ptr, ...)) expects (roller.py:545-550)
+    small_address = hip.DevicePtr(4096)
+    assert isinstance(small_address, int) and small_address + 16 == 4112
+    assert C.sizeof(hip._pack_arg(small_address)) == 8 and hip._pack_arg(small_address).value == 4096
+    assert hip._DataView(4096).ptr == 4096 and isinstance(hip._DataView(4096).ptr, hip.DevicePtr)
+    with hip.profiler_range("a range no profiler listens to"):
+        pass
     for small in (0, 7, -1, 2**31 - 1, np.int64(12)):
         packed = hip._pack_arg(small)
         assert isinstance(packed, C.c_int) and C.sizeof(packed) == 4      # a bare int is never a pointer
