@@ -390,7 +390,9 @@ class Policy:
 
         ``stream_k`` (default: the tile's own setting) estimates the stream-K kernel instead: every
         CU works grid / CUs tiles' worth of reduce steps, a fraction and not a whole number of
-        rounds, at a slightly lower efficiency and with a fixed cost for the pieces of split tiles."""
+        rounds, at a slightly lower efficiency, with a fixed cost, and with the time the last workgroup
+        of a tile needs to read the tile's pieces back (``stream_k_pieces`` of them at
+        ``stream_k_piece_bandwidth``: what makes small tiles win where K is long and M x N small)."""
         a, cfg = self.arch, self.matmul_config
         m, n = td.block_tile
         stream_k = td.stream_k if stream_k is None else stream_k
@@ -400,15 +402,41 @@ class Policy:
         tiles_per_cu = -(-td.grid_size // a.compute_max_core)
         resident = max(1, min(td.block_per_SM, stream_k if stream_k else tiles_per_cu))
         base, slope = a.mfma_efficiency
-        efficiency = base - slope * (1.0 / m + 1.0 / n) + (a.co_resident_gain if resident > 1 else 0.0)
-        efficiency = max((efficiency - (a.stream_k_loss if stream_k else 0.0)) * self.simd_balance(td.block_tile), 0.05)
+        x = 1.0 / m + 1.0 / n
+        efficiency = base - slope * x + (a.co_resident_gain if resident > 1 else 0.0)
+        # below the knee (tiles smaller than about 64 x 128) a reduce step is too short to cover its own
+        # barrier and round trips, and the efficiency leaves the line
+        efficiency -= a.small_tile_slope * max(0.0, x - a.small_tile_knee)
+        balance = self.simd_balance(td.block_tile)
+        efficiency = max((efficiency - (a.stream_k_loss if stream_k else 0.0)) * balance, 0.05)
         t_mfma = 2.0 * m * n * k_steps * td.rstep / (cu_flops * efficiency)
-        t_mem = td.traffic / cu_bw
-        t_fixed = a.tile_fixed_seconds + m * n * cfg.el_bytes / cu_bw
+        # a reduce step cannot be shorter than the round trip it hides (barrier, fragment reads, the
+        # next loads' issue); workgroups that share the CU take turns in it.  Only tiles of a few MFMA
+        # blocks get there.
+        t_mfma = max(t_mfma, k_steps * a.step_latency_seconds / resident)
+        # the tile's share of the operands has to come from device memory once; what the tiles read
+        # again comes from the caches, at ``cache_bandwidth_ratio`` times that rate
+        once = cfg.el_bytes * (cfg.M * cfg.K + cfg.K * cfg.N + cfg.M * cfg.N) / max(td.grid_size, 1)
+        t_mem = (min(once, td.traffic) + max(td.traffic - once, 0.0) / a.cache_bandwidth_ratio) / cu_bw
+        # filling the pipeline and draining the accumulators goes through the load and store ports of
+        # the SIMDs that hold the tile's waves: a three-wave tile takes 4/3 of the time (measured on
+        # 384 x 512 x 256: 48 x 16 tiles 4.4 us, 32 x 32 tiles 3.9 us)
+        t_fixed = (a.tile_fixed_seconds + m * n * cfg.el_bytes / cu_bw) / balance
         if stream_k:
             share = td.grid_size / a.compute_max_core          # tiles' worth of reduce steps per CU
-            return share * max(t_mfma, t_mem) + (-(-math.ceil(share) // resident) + 1) * t_fixed + a.stream_k_fixed_seconds
+            t_pieces = self.stream_k_pieces(td, stream_k) * m * n * cfg.el_bytes / (a.stream_k_piece_bandwidth * 1e9)
+            return share * max(t_mfma, t_mem) + (-(-math.ceil(share) // resident) + 1) * t_fixed + a.stream_k_fixed_seconds + t_pieces
         return tiles_per_cu * max(t_mfma, t_mem) + (-(-tiles_per_cu // resident)) * t_fixed
+
+    def stream_k_pieces(self, td: TileDict, stream_k: int) -> float:
+        """How many workgroups meet in one tile of a stream-K launch: with fewer reduce steps in a
+        share than in a tile, a tile's steps / a share's steps, plus one for the share that straddles
+        its start; otherwise two (a share ends inside at most one tile).  The workgroup that arrives last
+        reads that many pieces of the tile back, one after the other, which is what a split costs."""
+        k_steps = -(-self.matmul_config.K // td.rstep)
+        units = td.grid_size * k_steps
+        share = units / min(stream_k * self.arch.compute_max_core, units)
+        return k_steps / share + 1.0 if share < k_steps else 2.0
 
     def _choose_stream_k(self, td: TileDict) -> None:
         """Sets ``td.stream_k`` where the estimate says that working equal shares of reduce steps

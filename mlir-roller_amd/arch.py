@@ -58,6 +58,13 @@ class TileDevice:
     mfma_efficiency: Tuple[float, float] = (1.0, 0.0)
     co_resident_gain: float = 0.0
     tile_fixed_seconds: float = 0.0
+    # extra loss of issue efficiency per unit of (1/m + 1/n) beyond ``small_tile_knee``
+    small_tile_slope: float = 0.0
+    small_tile_knee: float = 1.0 / 64 + 1.0 / 128
+    # shortest time one reduce step of one workgroup can take, whatever its arithmetic (0 = no floor),
+    # and how much faster than device memory the caches deliver operand bytes that are read again
+    step_latency_seconds: float = 0.0
+    cache_bandwidth_ratio: float = 1.0
     # wave tiles of at most this many elements list the matrix instruction with the longer k first
     long_k_mfma_up_to: int = 0
     # whether the reduce step of a tile grows to what its share of workgroup memory allows (longer
@@ -72,6 +79,7 @@ class TileDevice:
     stream_k_workgroups: int = 0
     stream_k_loss: float = 0.0
     stream_k_fixed_seconds: float = 0.0
+    stream_k_piece_bandwidth: float = 1.0e9    # GB/s at which one workgroup reads the pieces of a split tile back
     stream_k_margin: float = 0.0
 
     def get_avaliable_tensorintrin_shapes(self) -> List[Tuple[int, int, int]]:
@@ -145,11 +153,18 @@ class MI355X(TileDevice):
     peak_matrix_tflops: float = 157.3
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
-    # (a test refits both): 0.978 for 256x256 tiles, 0.971 + 0.011 for 128x128 with two on a CU,
-    # 0.944 for 32x64
-    mfma_efficiency: Tuple[float, float] = (0.985, 0.87)
-    co_resident_gain: float = 0.011
+    # (a test refits them): 0.980 for 256x256 tiles, 0.975 + 0.007 for 128x128 with two on a CU,
+    # 0.970 + 0.007 for 64x128; below that knee the efficiency falls 2.5 per unit of (1/m + 1/n)
+    # faster (0.94 for 64x64, 0.89 for 32x64)
+    mfma_efficiency: Tuple[float, float] = (0.985, 0.63)
+    co_resident_gain: float = 0.007
+    small_tile_slope: float = 2.5
     tile_fixed_seconds: float = 1.0e-6
+    # chosen on the committed sweep, not fitted in closed form: 0.2-0.4 us and ratios of 2.5-4 rank
+    # its kernels identically (a test holds both ends); without the two, whole tiles of 32 x 32 lead on
+    # problems with a long K and few tiles, where they take twice the time of the best kernel
+    step_latency_seconds: float = 0.3e-6
+    cache_bandwidth_ratio: float = 3.0
     # 16x16x4 wins on every wave tile it fits (up to 64x128; a wave keeps at most 32 blocks), by
     # 0.5-2 % in the committed sweep
     long_k_mfma_up_to: int = 64 * 128
@@ -157,11 +172,13 @@ class MI355X(TileDevice):
     # second workgroup on the CU would use and lengthens the fill of the pipeline (measured: 128x128
     # tiles at K steps of 32 against 64, 64x64 at 32 / 64 / 128: the shortest wins or ties)
     grow_reduce_step: bool = False
-    # fitted like the constants above (stream-K against plain kernels of the same tile on problems that
-    # fill whole rounds: 0.9 % slower); about 5 us for the pieces of a launch
+    # fitted like the constants above: stream-K against plain kernels of the same tile on problems that
+    # fill whole rounds (0.7 % slower), and the rate at which the last workgroup of a tile that is split
+    # many ways reads the pieces back (30 GB/s: a round trip past the L2 each); about 5 us per launch besides
     stream_k_workgroups: int = 2
-    stream_k_loss: float = 0.009
+    stream_k_loss: float = 0.007
     stream_k_fixed_seconds: float = 5.0e-6
+    stream_k_piece_bandwidth: float = 30.0
     stream_k_margin: float = 0.02
     smem_cap: int = field(init=False)
     max_smem_usage: int = field(init=False)

@@ -44,12 +44,18 @@ SHAPES: Dict[str, Tuple[int, int, int]] = {f"M{i}": s for i, s in enumerate([
     (4096, 8192, 4096), (8192, 2048, 8192), (8192, 4096, 2048), (8192, 4096, 4096)])}
 SHAPES.update({"cfg4": (3000, 5000, 1536), "1024x1024x1024": (1024, 1024, 1024),
                "1536x1536x1536": (1536, 1536, 1536), "1000x1000x1000": (1000, 1000, 1000)})
-# ... small cubes, a tall and skinny problem, and two whose tile grids fill a fraction of their last round
+# ... small cubes, tall, wide and skinny problems, and two whose tile grids fill a fraction of their last round
 SHAPES.update({name: tuple(int(v) for v in name.split("x")) for name in (
-    "256x256x256", "512x512x512", "768x768x768", "65536x128x128", "2560x2560x2560", "1920x2880x2048")})
+    "256x256x256", "512x512x512", "768x768x768", "65536x128x128", "2560x2560x2560", "1920x2880x2048",
+    "384x512x256", "4096x64x4096", "64x4096x4096")})
 
 
 MIN_FIT_MS = 0.1   # shortest measurement the efficiency fit uses
+MIN_FIT_TILE = 64 * 128  # smallest block tile it uses: below, a reduce step is too short to hide its own round trips
+                         # and the efficiency falls away from the line (64 x 64: 0.90, 32 x 64: 0.87 where the line says 0.96)
+LEADERS = 1.03     # ... and how close to its shape's fastest kernel a record has to be
+WAVES_TIE = 0.005        # block sizes whose mean times differ by less are a tie
+INSTRUCTION_TIE = 0.002  # so are the two matrix instructions on a wave-tile size
 
 
 def shape_of(name: str) -> Tuple[int, int, int]:
@@ -135,18 +141,27 @@ def _solve(a: List[List[float]], b: List[float]) -> List[float]:
 def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
     """Least-squares ``efficiency = base - slope * (1/m + 1/n) + gain * [tiles share a CU]`` over
     the best record of every (shape, block tile) whose tile grid fills at least three quarters of
-    its last round of CUs (a sparse last round measures the tail, not the tile) and that ran for at
-    least ``MIN_FIT_MS`` (below that the launch itself is a visible share).  The gain is fitted
+    its last round of CUs (a sparse last round measures the tail, not the tile), that ran for at
+    least ``MIN_FIT_MS`` (below that the launch itself is a visible share), whose tile has at least
+    ``MIN_FIT_TILE`` elements, and that came within ``LEADERS`` of its shape's fastest kernel: the model
+    is asked to order the leaders of a shape, and how far behind an also-ran finishes (a 64 x 128 tile
+    on 8192 x 4096 x 4096 loses 4 % to cache misses that 1/m + 1/n does not describe) must not bend the
+    line -- nor should the fit depend on which also-rans a sweep happened to time.  The gain is fitted
     only when the records hold tiles of both kinds.  Deterministic: closed-form normal equations,
     records in sorted order."""
     arch = arch or MI355X()
+    fastest: Dict[tuple, float] = {}
+    for r in plain(records):
+        fastest[tuple(r["shape"])] = min(fastest.get(tuple(r["shape"]), float("inf")), r["ms"])
     xs, ys, zs = [], [], []
     for r in best_per_block_tile(records):
         M, N, _ = r["shape"]
         m, n = r["block_tile"]
+        if r["ms"] > LEADERS * fastest[tuple(r["shape"])]:
+            continue
         tiles = (-(-M // m)) * (-(-N // n))
         last_round = tiles % arch.compute_max_core or arch.compute_max_core
-        if M % m or N % n or last_round < 0.75 * arch.compute_max_core or r["ms"] < MIN_FIT_MS:
+        if M % m or N % n or last_round < 0.75 * arch.compute_max_core or r["ms"] < MIN_FIT_MS or m * n < MIN_FIT_TILE:
             continue
         eff = observed_efficiency(r, arch)
         if eff is None or not 0.3 < eff < 1.05:
@@ -168,6 +183,38 @@ def fit(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
             "rms_residual": math.sqrt(math.fsum(e * e for e in resid) / len(xs))}
 
 
+def fit_small_tiles(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
+    """How fast the efficiency leaves the line below the knee (``small_tile_slope``): over the best
+    record of every (shape, block tile) beyond ``arch.small_tile_knee`` that fills its last round and
+    ran for at least ``MIN_FIT_MS`` -- leaders or not: small tiles never lead where a kernel runs that
+    long -- a least-squares line through the knee of (line - observed efficiency) against
+    (1/m + 1/n - knee).  The line is the one ``fit`` gives for the same records."""
+    arch = arch or MI355X()
+    line = fit(records, arch)
+    xx = xy = 0.0
+    points = 0
+    for r in best_per_block_tile(records):
+        M, N, _ = r["shape"]
+        m, n = r["block_tile"]
+        x = 1.0 / m + 1.0 / n
+        tiles = (-(-M // m)) * (-(-N // n))
+        last_round = tiles % arch.compute_max_core or arch.compute_max_core
+        if x <= arch.small_tile_knee or M % m or N % n or last_round < 0.75 * arch.compute_max_core or r["ms"] < MIN_FIT_MS:
+            continue
+        eff = observed_efficiency(r, arch)
+        if eff is None or not 0.3 < eff < 1.05:
+            continue
+        together = min(resident_tiles(r, arch), -(-tiles // arch.compute_max_core)) > 1
+        expected = line["base"] - line["slope"] * x + (line["gain"] if together else 0.0)
+        dx = x - arch.small_tile_knee
+        xx += dx * dx
+        xy += dx * (expected - eff)
+        points += 1
+    if points < 5:
+        raise ValueError(f"only {points} block tiles below the knee; need at least 5")
+    return {"small_tile_slope": round(max(xy / xx, 0.0), 1), "points": points}
+
+
 def _geo_mean(ratios: Sequence[float]) -> float:
     return math.exp(math.fsum(math.log(r) for r in ratios) / len(ratios))
 
@@ -175,7 +222,9 @@ def _geo_mean(ratios: Sequence[float]) -> float:
 def fit_waves_per_simd(records: Sequence[dict], arch: Optional[TileDevice] = None, min_tile: int = 128 * 128) -> dict:
     """Which block size the recommendation should try first: for every (shape, block tile) of at
     least ``min_tile`` elements measured both with one and with two waves per SIMD, the ratio of
-    the two best times; the geometric mean over all pairs decides (``waves_per_partition``)."""
+    the two best times; the geometric mean over all pairs decides (``waves_per_partition``): two
+    waves only where they win by more than ``WAVES_TIE`` -- within that, a coin that re-measuring
+    would flip, the smaller block (larger wave tiles, fewer operand reads per FLOP) stays first."""
     arch = arch or MI355X()
     one, two = arch.warp_size * arch.sm_partition, 2 * arch.warp_size * arch.sm_partition
     best: Dict[tuple, Dict[int, float]] = {}
@@ -188,14 +237,15 @@ def fit_waves_per_simd(records: Sequence[dict], arch: Optional[TileDevice] = Non
     if not ratios:
         raise ValueError("no block tile was measured at both block sizes")
     mean = _geo_mean(ratios)
-    return {"waves_per_partition": 1 if mean >= 1.0 else 2, "two_over_one": mean, "pairs": len(ratios)}
+    return {"waves_per_partition": 1 if mean >= 1.0 - WAVES_TIE else 2, "two_over_one": mean, "pairs": len(ratios)}
 
 
 def fit_long_k_mfma(records: Sequence[dict], arch: Optional[TileDevice] = None) -> dict:
     """Up to which wave-tile size the instruction with the longer k (16x16x4) should be listed
     first: for every wave-tile size, the geometric mean of time(32x32x2) / time(16x16x4) over the
     (shape, block tile, wave tile) triples measured with both; the largest size whose mean is
-    above 1, with every smaller size above 1 as well (``long_k_mfma_up_to``)."""
+    above ``1 - INSTRUCTION_TIE``, with every smaller size above it as well (``long_k_mfma_up_to``;
+    a tie keeps the instruction that wins on the smaller wave tiles)."""
     by: Dict[tuple, Dict[int, float]] = {}
     for r in plain(records):
         key = (tuple(r["shape"]), tuple(r["block_tile"]), tuple(r["wave_tile"]))
@@ -208,7 +258,7 @@ def fit_long_k_mfma(records: Sequence[dict], arch: Optional[TileDevice] = None) 
     means = {size: _geo_mean(v) for size, v in sorted(per_size.items())}
     up_to = 0
     for size, mean in means.items():
-        if mean <= 1.0:
+        if mean <= 1.0 - INSTRUCTION_TIE:
             break
         up_to = size
     return {"long_k_mfma_up_to": up_to, "mi32_over_mi16_by_wave_tile_elems": {k: round(v, 4) for k, v in means.items()},
@@ -217,8 +267,10 @@ def fit_long_k_mfma(records: Sequence[dict], arch: Optional[TileDevice] = None) 
 
 def fit_stream_k(records: Sequence[dict], arch: Optional[TileDevice] = None, min_ms: float = 0.25) -> dict:
     """What the stream-K form of a kernel costs where it has nothing to gain: over every kernel
-    measured in both forms on a problem whose tile grid fills whole rounds of CUs and that runs for
-    at least ``min_ms``, the geometric mean of time(stream-K) / time(plain), minus one
+    measured in both forms on a problem whose tile grid fills whole rounds of CUs, that runs for
+    at least ``min_ms`` and whose tile has at least ``MIN_FIT_TILE`` elements (smaller tiles pay the
+    walk from segment to segment more often, and how many of them a sweep holds should not move the
+    figure), the geometric mean of time(stream-K) / time(plain), minus one
     (``stream_k_loss``).  Per shape, the best plain time over the best stream-K time is listed for the
     record (above 1: a stream-K kernel is the fastest one measured)."""
     arch = arch or MI355X()
@@ -235,12 +287,43 @@ def fit_stream_k(records: Sequence[dict], arch: Optional[TileDevice] = None, min
             slot = best.setdefault(shape, {})
             slot[form] = min(slot.get(form, float("inf")), ms)
         tiles = (-(-shape[0] // tile[0])) * (-(-shape[1] // tile[1]))
-        if 0 in t and 1 in t and tiles % arch.compute_max_core == 0 and t[0] >= min_ms:
+        if 0 in t and 1 in t and tiles % arch.compute_max_core == 0 and t[0] >= min_ms and tile[0] * tile[1] >= MIN_FIT_TILE:
             whole.append(t[1] / t[0])
     if not whole:
         raise ValueError("no kernel was measured in both forms on a problem that fills whole rounds")
     gains = {"x".join(str(v) for v in shape): round(t[0] / t[1], 4) for shape, t in sorted(best.items()) if 0 in t and 1 in t}
     return {"stream_k_loss": round(_geo_mean(whole) - 1.0, 3), "pairs": len(whole), "best_plain_over_best_stream_k": gains}
+
+
+def fit_stream_k_pieces(records: Sequence[dict], arch: Optional[TileDevice] = None, min_pieces: float = 6.0,
+                        depth: int = DEFAULT_PIPELINE_DEPTH) -> dict:
+    """The rate at which the last workgroup of a split tile gets the tile's pieces back
+    (``stream_k_piece_bandwidth``, GB/s): over the stream-K kernels whose tiles are split
+    ``min_pieces`` ways or more -- long K, few tiles -- a least-squares line through the origin of
+    (measured time - the estimate without that term) against the bytes of pieces read per tile."""
+    import dataclasses
+
+    arch = arch or MI355X()
+    free = dataclasses.replace(arch, stream_k_piece_bandwidth=1.0e12)   # the term switched off
+    xx = xy = 0.0
+    points = 0
+    for r in records:
+        if not r.get("stream_k"):
+            continue
+        cfg = MatmulConfig(*r["shape"], 32)
+        policy = Policy(cfg, free, depth)
+        td = TileDict.from_block_tile(list(r["block_tile"]), r["rstep"], cfg, free, depth)
+        pieces = policy.stream_k_pieces(td, r["stream_k"])
+        if pieces < min_pieces:
+            continue
+        x = pieces * r["block_tile"][0] * r["block_tile"][1] * cfg.el_bytes
+        y = r["ms"] * 1e-3 - policy.estimate_seconds(td, r["stream_k"])
+        xx += x * x
+        xy += x * y
+        points += 1
+    if points < 8 or xy <= 0.0:
+        raise ValueError("too few heavily split stream-K kernels in the data to fit the piece bandwidth")
+    return {"stream_k_piece_bandwidth": float(f"{xx / xy / 1e9:.2g}"), "points": points}
 
 
 # ---------------------------------------------------------------------------------------------
@@ -361,6 +444,22 @@ def measure(shape_names: Sequence[str], topk: int, depth: int = DEFAULT_PIPELINE
             "records": records}
 
 
+def merge(data: dict, earlier: dict) -> dict:
+    """Two sessions of the same sweep as one data set: the union of their kernels, each with the
+    shortest time either session measured for it."""
+    def key(r: dict) -> tuple:
+        return (tuple(r["shape"]), tuple(r["block_tile"]), tuple(r["wave_tile"]), r["mfma"], r["rstep"], r["threads"], r.get("stream_k", 0))
+    best = {key(r): r for r in earlier["records"]}
+    for r in data["records"]:
+        if key(r) not in best or r["ms"] < best[key(r)]["ms"]:
+            best[key(r)] = r
+    out = dict(data)
+    out["records"] = sorted(best.values(), key=lambda r: (list(SHAPES.values()).index(tuple(r["shape"])) if tuple(r["shape"]) in SHAPES.values() else len(SHAPES),
+                                                          r["shape"], r["rank_when_measured"], r["block_tile"], r["wave_tile"], r["mfma"], r.get("stream_k", 0)))
+    out["sessions"] = data.get("sessions", 1) + earlier.get("sessions", 1)
+    return out
+
+
 def load(path: Path = DEFAULT_DATA) -> dict:
     return json.loads(Path(path).read_text())
 
@@ -372,6 +471,8 @@ def main(argv=None) -> int:
     m.add_argument("--out", default=str(DEFAULT_DATA))
     m.add_argument("--topk", type=int, default=96, help="kernels per shape, both forms (whole tiles and stream-K) counted")
     m.add_argument("--shapes", nargs="*", default=list(SHAPES))
+    m.add_argument("--merge", nargs="*", default=[], help="earlier data sets of the same sweep: per kernel the shortest time of all "
+                   "sessions is kept (a session's slow outliers -- a busy neighbour, a cold cache -- drop out)")
     pc = sub.add_parser("precompile", help="no GPU: fill the code-object cache with the kernels that `measure` will time")
     pc.add_argument("--topk", type=int, default=96)
     pc.add_argument("--shapes", nargs="*", default=list(SHAPES))
@@ -400,6 +501,9 @@ def main(argv=None) -> int:
         return 1 if failed else 0
     if args.cmd == "measure":
         data = measure(args.shapes, args.topk)
+        data["sessions"] = 1
+        for earlier in args.merge:
+            data = merge(data, load(Path(earlier)))
         out = Path(args.out)
         out.parent.mkdir(parents=True, exist_ok=True)
         out.write_text(json.dumps(data, separators=(",", ":")).replace('},{"shape"', '},\n{"shape"'))
@@ -420,6 +524,17 @@ def main(argv=None) -> int:
                   f"{now.stream_k_loss}; best plain over best stream-K per shape: {sk['best_plain_over_best_stream_k']}")
         except ValueError as e:
             print(f"stream_k_loss not fitted: {e}")
+        try:
+            pc = fit_stream_k_pieces(data["records"])
+            print(f"fitted stream_k_piece_bandwidth = {pc['stream_k_piece_bandwidth']} GB/s ({pc['points']} heavily split kernels); "
+                  f"arch.MI355X has {now.stream_k_piece_bandwidth}")
+        except ValueError as e:
+            print(f"stream_k_piece_bandwidth not fitted: {e}")
+        try:
+            small = fit_small_tiles(data["records"])
+            print(f"fitted small_tile_slope = {small['small_tile_slope']} ({small['points']} block tiles below the knee); arch.MI355X has {now.small_tile_slope}")
+        except ValueError as e:
+            print(f"small_tile_slope not fitted: {e}")
         instr = fit_long_k_mfma(data["records"])
         print(f"fitted long_k_mfma_up_to = {instr['long_k_mfma_up_to']} (32x32x2 over 16x16x4 by wave-tile elements: "
               f"{instr['mi32_over_mi16_by_wave_tile_elems']}); arch.MI355X has {now.long_k_mfma_up_to}")

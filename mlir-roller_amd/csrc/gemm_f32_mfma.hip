@@ -927,25 +927,44 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const unsigned before = __builtin_amdgcn_readfirstlane(__builtin_bit_cast(unsigned, lds[0]));
     store_c = before == pieces - 1;
     if (store_c) {
-      auto add_piece = [&](auto is_first, unsigned slot) __attribute__((always_inline)) {
-        const __amdgpu_buffer_rsrc_t rr = make_rsrc(sk_slots + (long)slot * (BM * BN), (long)BM * BN * 4);
+      // One row of MFMA blocks at a time, the pieces of that row in K order.  The loads of up to
+      // AHEAD pieces are in flight together (every one is a round trip past the L2, and one after the
+      // other they made a tile of many pieces wait for each in turn); AHEAD keeps them within 32
+      // registers, and a row at a time keeps the kernel at two waves per SIMD (left alone, the
+      // scheduler issues every load of a piece first and needs a second set of accumulators).
+      constexpr int ROW_CHUNKS = TN * CHUNKS;
+      constexpr int AHEAD = ROW_CHUNKS <= 2 ? 4 : ROW_CHUNKS <= 4 ? 2 : 1;
 #pragma unroll
-        for (int bi = 0; bi < TM; ++bi) {
+      for (int bi = 0; bi < TM; ++bi) {
+        for (unsigned p0 = 0; p0 < pieces; p0 += AHEAD) {
+          v4f v[AHEAD][ROW_CHUNKS];
 #pragma unroll
-          for (int bj = 0; bj < TN; ++bj)
+          for (int a = 0; a < AHEAD; ++a) {
+            // past the last piece: the last one again (loaded, not added)
+            const unsigned piece = p0 + a < pieces ? p0 + a : pieces - 1;
+            const unsigned slot = piece == 0 ? 2 * first_wg + 1 : 2 * (first_wg + piece);
+            const __amdgpu_buffer_rsrc_t rr = make_rsrc(sk_slots + (long)slot * (BM * BN), (long)BM * BN * 4);
 #pragma unroll
-            for (int c = 0; c < CHUNKS; ++c) {
-              const v4f v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, SK_COHERENT));
+            for (int bj = 0; bj < TN; ++bj)
 #pragma unroll
-              for (int e = 0; e < 4; ++e) acc[bi][bj][4 * c + e] = decltype(is_first)::value ? v[e] : acc[bi][bj][4 * c + e] + v[e];
+              for (int c = 0; c < CHUNKS; ++c)
+                v[a][bj * CHUNKS + c] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rr, (unsigned)((((bi * TN + bj) * CHUNKS + c) * NT + tid) * 16), 0, SK_COHERENT));
+          }
+#pragma unroll
+          for (int a = 0; a < AHEAD; ++a) {
+            if (p0 + a < pieces) {               // the same for every lane
+#pragma unroll
+              for (int bj = 0; bj < TN; ++bj)
+#pragma unroll
+                for (int c = 0; c < CHUNKS; ++c)
+#pragma unroll
+                  for (int e = 0; e < 4; ++e)
+                    acc[bi][bj][4 * c + e] = p0 + a == 0 ? v[a][bj * CHUNKS + c][e] : acc[bi][bj][4 * c + e] + v[a][bj * CHUNKS + c][e];
             }
-          // one row of blocks at a time: left alone, the scheduler issues every load of the piece first and
-          // the kernel needs a second set of accumulator registers for them (one wave per SIMD instead of two)
+          }
           __builtin_amdgcn_sched_barrier(0);
         }
-      };
-      add_piece(int_c<1>{}, 2 * first_wg + 1);
-      for (unsigned piece = 1; piece < pieces; ++piece) add_piece(int_c<0>{}, 2 * (first_wg + piece));
+      }
       if (tid == 0) __hip_atomic_store(&sk_arrivals[seg.tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }

@@ -404,20 +404,48 @@ def test_committed_ranking_constants_equal_a_refit_of_the_committed_sweep():
     assert calibrate.fit_long_k_mfma(records)["long_k_mfma_up_to"] == arch.long_k_mfma_up_to
     stream_k = calibrate.fit_stream_k(records)
     assert stream_k["stream_k_loss"] == arch.stream_k_loss and stream_k["pairs"] >= 100, stream_k
+    pieces = calibrate.fit_stream_k_pieces(records)
+    assert pieces["stream_k_piece_bandwidth"] == arch.stream_k_piece_bandwidth and pieces["points"] >= 50, pieces
+    small = calibrate.fit_small_tiles(records)
+    assert small["small_tile_slope"] == arch.small_tile_slope and small["points"] >= 10, small
     from mlir_roller_amd.benchmark import README_SHAPES
     rows = {tuple(r["shape"]): r for r in calibrate.check(records, topk=4)}
     for shape in list(README_SHAPES) + [(3000, 5000, 1536)]:
         row = rows[shape]
         assert row["unmeasured_in_topk"] == 0 and row["topk_over_fastest"] <= 1.01, row
         assert row["top1_over_fastest"] <= 1.02, row
-    # off the benchmark table -- cubes from 256 to 2560, a problem of one and a half rounds of tiles: the
-    # first four hints stay within 2.5 % of the fastest kernel measured (the first hint alone does not on
-    # the smallest cube).  The tall and skinny 65536 x 128 x 128 (four K steps per tile) is the known
-    # outlier: 9 % off, the fastest kernel there being one that the tile ranking puts far down
-    for shape, row in rows.items():
-        if shape not in README_SHAPES and shape != (65536, 128, 128):
-            assert row["unmeasured_in_topk"] == 0 and row["topk_over_fastest"] <= 1.025, row
-    assert rows[(65536, 128, 128)]["topk_over_fastest"] <= 1.10
+    # off the benchmark table -- cubes from 512 to 2560, a problem of one and a half rounds of tiles, problems
+    # with a long K and few tiles (where a stream-K kernel is twice as fast as any whole-tile kernel):
+    # the first four hints hold a kernel within 1 % of the fastest measured.  Two outliers are known: the
+    # smallest cube, a 3.7 us kernel whose leaders differ by less than the launch-to-launch spread, and the tall
+    # and skinny 65536 x 128 x 128 (four K steps per tile), whose fastest kernels have eight waves
+    off_table = [s for s in rows if s not in README_SHAPES and s != (3000, 5000, 1536)]
+    assert {(4096, 64, 4096), (64, 4096, 4096), (384, 512, 256), (256, 256, 256), (65536, 128, 128)} <= set(off_table)
+    for shape in off_table:
+        limit = {(256, 256, 256): 1.05, (65536, 128, 128): 1.05}.get(shape, 1.01)
+        assert rows[shape]["unmeasured_in_topk"] == 0 and rows[shape]["topk_over_fastest"] <= limit, rows[shape]
+    # a stream-K kernel leads where K is long and the tiles are few, and there the first hint is the fastest
+    for shape in [(4096, 64, 4096), (64, 4096, 4096)]:
+        assert stream_k["best_plain_over_best_stream_k"]["x".join(map(str, shape))] > 1.8
+        assert rows[shape]["top1_over_fastest"] <= 1.01, rows[shape]
+
+
+def test_the_latency_and_cache_terms_of_the_estimate_matter_where_k_is_long_and_tiles_are_few():
+    """``step_latency_seconds`` and ``cache_bandwidth_ratio`` are not fitted in closed form but chosen on
+    the committed sweep; this pins what they are for.  With both switched off the first four hints of
+    4096 x 64 x 4096 miss the fastest measured kernel by more than 5 %; with the committed values, and
+    with any values in the ranges named beside them, they hold it."""
+    import dataclasses
+    from mlir_roller_amd import calibrate
+    records = [r for r in calibrate.load()["records"] if tuple(r["shape"]) in {(4096, 64, 4096), (64, 4096, 4096)}]
+
+    def worst(arch):
+        return max(1e9 if row["topk_over_fastest"] is None else row["topk_over_fastest"] for row in calibrate.check(records, arch=arch, topk=4))
+    base = MI355X()
+    assert worst(base) <= 1.01
+    assert worst(dataclasses.replace(base, step_latency_seconds=0.0, cache_bandwidth_ratio=1.0)) > 1.05
+    for latency, ratio in ((0.2e-6, 2.5), (0.4e-6, 4.0)):
+        assert worst(dataclasses.replace(base, step_latency_seconds=latency, cache_bandwidth_ratio=ratio)) <= 1.01, (latency, ratio)
 
 
 def test_ranking_model_holds_on_a_shape_it_was_not_fitted_on():

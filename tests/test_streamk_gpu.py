@@ -63,6 +63,13 @@ CASES = [
     (GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 4, 1, 0, 8, 0, 1, 0, 2), [(1000, 1000, 1000)]),
     (GemmConfig(128, 64, 32, 64, 32, 16, 3, 0, 0, 4, 2, 2, 3, 0, 1, 0, 4), [(1100, 900, 512)]),
     (GemmConfig(64, 64, 32, 32, 32, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1, 0, 8), [(1000, 1000, 1000), (70, 92, 52)]),
+    # few tiles and a long K: every tile is split five to sixty-four ways, and the workgroup that arrives last
+    # reads the pieces back four, two or one at a time (two, four or sixteen 16-byte chunks per row of blocks)
+    (GemmConfig(64, 32, 32, 16, 32, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2), [(4096, 64, 4096), (256, 128, 2048), (256, 128, 1216), (256, 128, 1120)]),   # 4, 32, 19/37/38, 18/22/35 pieces
+    (GemmConfig(32, 64, 32, 16, 32, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2), [(64, 4096, 4096)]),
+    (GemmConfig(64, 64, 32, 32, 32, 16, 3, 0, 0, 4, 2, 3, 8, 0, 1, 0, 2), [(4096, 64, 4096), (250, 132, 2048 + 32)]),
+    (GemmConfig(128, 64, 32, 32, 64, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2), [(4096, 64, 4096)]),
+    (GemmConfig(64, 64, 32, 32, 32, 32, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 1), [(512, 512, 8192)]),
 ]
 FLAT = [(cfg, shape) for cfg, shapes in CASES for shape in shapes]
 
