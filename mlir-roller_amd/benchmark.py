@@ -40,9 +40,13 @@ README_SHAPES: List[Tuple[int, int, int]] = [
 ]
 
 
-# Off the headline table: the ragged named configuration and cubes that put one small tile on a CU
+# Off the headline table: the ragged named configuration, cubes that put one small tile on a CU, two
+# problems whose tiles fill a fraction of their last round of CUs, and problems with a long K and few
+# tiles (the last two kinds are where the stream-K kernels lead)
 MID_SHAPES: List[Tuple[int, int, int]] = [(3000, 5000, 1536), (1024, 1024, 1024), (1000, 1000, 1000), (1536, 1536, 1536),
-                                          (1024, 4096, 1024), (16384, 1024, 1024), (6144, 6144, 6144)]
+                                          (1024, 4096, 1024), (16384, 1024, 1024), (6144, 6144, 6144),
+                                          (2560, 2560, 2560), (1920, 2880, 2048), (4096, 64, 4096), (64, 4096, 4096),
+                                          (512, 512, 8192), (65536, 128, 128)]
 
 
 def benchmark(test_shapes: Sequence[Tuple[int, int, int]], topk: int = DEFAULT_TOPK,
