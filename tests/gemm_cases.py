@@ -84,3 +84,36 @@ def seeded_template_cases(count: int = 72, seed: int = TEMPLATE_SEEDS[0]):
             continue
         yield case, cfg, (M, N, K)
         case += 1
+
+
+STREAMK_SEED = 20250911
+
+
+def seeded_streamk_cases(count: int = 48, seed: int = STREAMK_SEED):
+    """Yields ``(case, GemmConfig, (M, N, K))``: the draw of ``seeded_template_cases`` (another seed)
+    moved onto the stream-K form of the kernel -- the pipelined loop on two buffers, 1, 2 or 4
+    workgroups per CU -- with K lengthened to 3-40 K steps, so that tiles are split from two to
+    dozens of ways.  Only configurations that ``rl_gemm_config_check`` accepts are kept."""
+    import dataclasses
+
+    from mlir_roller_amd import hip
+
+    rng = np.random.default_rng(seed + 1)
+    case = 0
+    for _, cfg, (M, N, K) in seeded_template_cases(count=4 * count, seed=seed):
+        if case == count:
+            break
+        sk = dataclasses.replace(cfg, stages=3, streamk=int(rng.choice([1, 2, 2, 4])))
+        steps = int(rng.integers(3, 41))
+        K = (steps - 1) * cfg.bk + (K - 1) % cfg.bk + 1          # the drawn remainder of the last K step is kept
+        if cfg.vec == 4:
+            K = max(4, K // 4 * 4)
+        if cfg.edge != 1 and K % cfg.bk:
+            K = -(-K // cfg.bk) * cfg.bk
+        try:
+            hip.config_check(sk)
+        except hip.HipError:
+            continue
+        yield case, sk, (M, N, K)
+        case += 1
+

@@ -92,6 +92,28 @@ def test_streamk_matches_oracle_within_tolerance_and_exactly_on_integers(device,
         assert np.array_equal(first.view(np.uint32), run(cfg, A, B).view(np.uint32))   # same bits whoever arrives last
 
 
+def test_seeded_points_of_the_template_parameter_space_are_exact_as_stream_k(device):
+    """Forty-eight seeded (configuration, shape) pairs from everything the configuration check accepts with
+    ``streamk`` set -- both instructions, 1 to 8 waves, 1 to 7 column blocks per wave, both operand layouts,
+    every edge mode, access width, remap mode and padding -- on integer inputs: bit-exact against the oracle, in
+    overwrite and in accumulate mode, whatever way the split falls."""
+    sys.path.insert(0, str(__import__("pathlib").Path(__file__).resolve().parent))
+    from gemm_cases import seeded_streamk_cases
+    seen = set()
+    for case, cfg, (M, N, K) in seeded_streamk_cases():
+        sched = hip.streamk_schedule(cfg, M, N, K, device.compute_units)
+        say("stream-K template case", case, cfg.tag(), (M, N, K), "grid", sched.grid, "tiles", sched.tiles, "K steps", sched.k_steps)
+        A, B = go.make_inputs(M, N, K, seed=3000 + case, distribution="integer")
+        want = go.gemm_f32(A, B)
+        if cfg.accum:
+            C0 = np.random.default_rng(case).integers(0, 10, (M, N)).astype(np.float32)
+            assert np.array_equal(run(cfg, A, B, c_init=C0), want + C0), (case, cfg.tag(), (M, N, K))
+        else:
+            assert np.array_equal(run(cfg, A, B), want), (case, cfg.tag(), (M, N, K))
+        seen.add((cfg.mi, cfg.edge, cfg.vec, cfg.direct, cfg.trans_b, cfg.streamk))
+    assert len(seen) >= 30          # the draw really spreads over the parameter space
+
+
 def test_streamk_accumulates_into_c(device):
     cfg = GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 4, 1, 3, 8, 1, 1, 0, 2)
     M, N, K = 300, 260, 512
