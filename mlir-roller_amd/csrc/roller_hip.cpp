@@ -473,7 +473,9 @@ int workspace_for(hipStream_t stream, size_t bytes, void** out) {
     }
     const size_t want = bytes + bytes / 4;   // head room, so that a slightly larger problem does not reallocate
     HIP_TRY(hipMalloc(&w.ptr, want));
-    HIP_TRY(hipMemset(w.ptr, 0, want));
+    // zeroed on the launch stream itself: in order with the kernel that follows, also on a stream
+    // that does not synchronise with the default stream
+    HIP_TRY(hipMemsetAsync(w.ptr, 0, want, stream));
     w.bytes = want;
   }
   *out = w.ptr;

@@ -467,10 +467,28 @@ def test_ranking_model_holds_on_a_shape_it_was_not_fitted_on():
         assert row["topk_over_fastest"] is not None and row["topk_over_fastest"] <= 1.03, (shape, fit["mfma_efficiency"], row)
 
 
+def test_sessions_of_a_sweep_merge_to_the_shortest_time_per_kernel():
+    from mlir_roller_amd import calibrate
+    rec = lambda tile, ms, sk=0, rank=1: {"shape": [2048, 2048, 2048], "block_tile": list(tile), "wave_tile": [32, 64], "mfma": 16, "rstep": 32,
+                                          "threads": 256, "edge": 0, "direct": 1, "stream_k": sk, "rank_when_measured": rank, "ms": ms}
+    first = {"device": {}, "records": [rec((64, 128), 0.120), rec((128, 128), 0.119, rank=2), rec((64, 128), 0.125, sk=2, rank=3)]}
+    second = {"device": {}, "sessions": 2, "records": [rec((64, 128), 0.117), rec((128, 128), 0.121, rank=2), rec((128, 64), 0.118, rank=4)]}
+    both = calibrate.merge(first, second)
+    assert both["sessions"] == 3
+    got = {(tuple(r["block_tile"]), r["stream_k"]): r["ms"] for r in both["records"]}
+    assert got == {((64, 128), 0): 0.117, ((128, 128), 0): 0.119, ((64, 128), 2): 0.125, ((128, 64), 0): 0.118}
+    assert [r["rank_when_measured"] for r in both["records"]] == [1, 2, 3, 4]         # in the order of the sweep
+
+
 def test_refit_rejects_a_sweep_that_cannot_pin_the_model():
     from mlir_roller_amd import calibrate
     with pytest.raises(ValueError):
         calibrate.fit([])
+    big_tiles_only = [r for r in calibrate.load()["records"] if min(r["block_tile"]) >= 128]
+    with pytest.raises(ValueError):
+        calibrate.fit_small_tiles(big_tiles_only)            # nothing below the knee
+    with pytest.raises(ValueError):
+        calibrate.fit_stream_k_pieces([r for r in big_tiles_only if tuple(r["shape"]) == (4096, 8192, 4096)])   # no tile split many ways
     one = [{"shape": [4096, 4096, 4096], "block_tile": [256, 256], "wave_tile": [128, 128], "mfma": 32, "rstep": 32,
             "threads": 256, "ms": 0.95}]
     with pytest.raises(ValueError):
