@@ -50,6 +50,7 @@ SHAPES.update({name: tuple(int(v) for v in name.split("x")) for name in (
     "384x512x256", "4096x64x4096", "64x4096x4096")})
 
 
+SETTLE_MS = 15.0   # run-up of every kernel ahead of its timed launches (the clocks follow the load, see tuner.time_candidates)
 MIN_FIT_MS = 0.1   # shortest measurement the efficiency fit uses
 MIN_FIT_TILE = 64 * 128  # smallest block tile it uses: below, a reduce step is too short to hide its own round trips
                          # and the efficiency falls away from the line (64 x 64: 0.90, 32 x 64: 0.87 where the line says 0.96)
@@ -428,7 +429,7 @@ def measure(shape_names: Sequence[str], topk: int, depth: int = DEFAULT_PIPELINE
                 say(f"[calibrate] {name} hint {rank} skipped: {e}")
         for i in range(0, len(cands), chunk):
             part = cands[i:i + chunk]
-            times = time_candidates([c[3] for c in part], bufs, shape, stream=stream)
+            times = time_candidates([c[3] for c in part], bufs, shape, stream=stream, settle_ms=SETTLE_MS)
             for (rank, hint, g, _), ms in zip(part, times):
                 records.append({"shape": list(shape), "block_tile": list(hint.block_tile), "wave_tile": list(hint.wave_tile),
                                 "mfma": hint.mfma, "rstep": hint.rstep, "threads": hint.threads, "edge": g.edge,
@@ -440,7 +441,7 @@ def measure(shape_names: Sequence[str], topk: int, depth: int = DEFAULT_PIPELINE
             b.free()
     return {"device": {"name": props.name.decode(), "arch": props.arch.decode(), "compute_units": props.compute_units,
                        "clock_khz": props.clock_khz},
-            "pipeline_depth": depth, "protocol": "per kernel: best of 2 alternating batches of 8 launches behind a 40 ms clock ramp, HIP events on the launch stream",
+            "pipeline_depth": depth, "protocol": "per kernel: best of 2 alternating batches of 8 launches, each behind 15 ms of the same kernel, behind a 40 ms clock ramp; HIP events on the launch stream",
             "records": records}
 
 

@@ -16,6 +16,7 @@ stream with the engine-clock ramp queued ahead of the timed launches.
 
 from __future__ import annotations
 
+import math
 from typing import List, Optional, Sequence, Tuple
 
 DEFAULT_TOPK = 4      # hints tried per shape (the reference: 20, benchmark.py:10)
@@ -47,13 +48,19 @@ def ramp_launches(shape: Tuple[int, int, int], at_least: int = 0) -> int:
 
 
 def time_candidates(plans: Sequence, bufs, shape: Tuple[int, int, int], stream=None, reps: int = 8,
-                    rounds: int = 2, gap_launches: int = 2) -> List[float]:
+                    rounds: int = 2, gap_launches: int = 2, settle_ms: float = 0.0) -> List[float]:
     """Milliseconds per launch for each plan in ``plans`` (objects with ``launch(A, B, C, M, N, K,
     stream=)``), all measured behind ONE clock ramp and with no host synchronisation in between:
     a synchronisation (or the host loading the next module) between candidates would idle the
     GPU and put the next measurement into the ramp again.  Every candidate is timed ``rounds``
     times in alternation with the others and its best mean is returned, which takes slow drifts
-    (temperature, clock) out of the comparison."""
+    (temperature, clock) out of the comparison.
+
+    ``settle_ms``: untimed launches of a candidate, worth that many milliseconds, ahead of each of its
+    timed batches.  The clocks follow the load: after 20 ms of a kernel that keeps half of the SIMDs
+    busy, a full-rate kernel ran 12 % slow and needed 14 ms to recover (measured), so a sweep that
+    mixes good and poor kernels gives every candidate its own run-up; the policy's first hints are
+    all full-rate kernels and need none."""
     from . import hip
     from .hip import Event
 
@@ -63,10 +70,11 @@ def time_candidates(plans: Sequence, bufs, shape: Tuple[int, int, int], stream=N
     launch = lambda plan: plan.launch(bufs[0], bufs[1], bufs[2], M, N, K, stream=stream)
     for _ in range(ramp_launches(shape)):
         launch(plans[0])
+    run_up = max(gap_launches, math.ceil(ramp_launches(shape) * settle_ms / RAMP_MS)) if settle_ms > 0 else gap_launches
     marks = []
     for _ in range(max(rounds, 1)):
         for i, plan in enumerate(plans):
-            for _ in range(gap_launches):
+            for _ in range(run_up):
                 launch(plan)
             e0, e1 = Event(), Event()
             e0.record(stream)

@@ -289,11 +289,13 @@ def test_mi355x_block_sizes_aim_for_one_wave_per_simd():
     assert policy.score_block_size(192) > policy.score_block_size(512)  # three waves leave a SIMD idle
     assert Policy(cfg, CUDA()).recommend_block_size(TileDict.from_block_tile([128, 128], 32, cfg, CUDA()))[0] == 128
     hints = get_roller_hints(cfg, MI355X(), topk=4)
-    # one hint per block tile, at one wave per SIMD, with the 16x16x4 instruction.  First the tile of
-    # which two fit a CU at once (each hides the other's barriers, fill and drain)
+    # one hint per block tile, at one wave per SIMD, with the 16x16x4 instruction where it fits.  First the
+    # tile of which two fit a CU at once (each hides the other's barriers, fill and drain), then its
+    # neighbours of the same kind, then the one-per-CU tile with the 32x32x2 instruction
     assert [(h.block_tile, h.wave_tile, h.threads, h.mfma, h.stream_k) for h in hints] == [
         ([128, 128], [64, 64], 256, 16, 0), ([64, 256], [64, 64], 256, 16, 0),
-        ([256, 64], [64, 64], 256, 16, 0), ([64, 128], [32, 64], 256, 16, 0)]
+        ([256, 64], [64, 64], 256, 16, 0), ([256, 256], [128, 128], 256, 32, 0)]
+    assert len({tuple(h.block_tile) for h in hints}) == 4
     # the second block size of a tile is still there for callers that complete tiles themselves
     td = policy.get_block_tiles_candidates([1, 1], 32)[0]
     assert [(h.wave_tile, h.threads) for h in policy.assign_thread_tile(td, 2)] == [([64, 64], 256), ([32, 64], 512)]
