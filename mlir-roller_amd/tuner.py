@@ -22,6 +22,8 @@ from typing import List, Optional, Sequence, Tuple
 DEFAULT_TOPK = 4      # hints tried per shape (the reference: 20, benchmark.py:10)
 TIE_MARGIN = 0.01     # relative spread of two timings of the same kernel: about half a percent a few milliseconds
                       # apart, up to three percent for small-tile kernels between one batch of launches and the next
+PICK_SETTLE_MS = 2.0  # run-up of each candidate ahead of its timed launches when the tuner compares hints (a long
+                      # list, as the reference's top-20, holds kernels of very different load)
 RAMP_MS = 40.0        # continuous load queued ahead of a timed region: the engine clock drops within
                       # microseconds of the GPU going idle and needs about 25 ms to come back
 
@@ -92,7 +94,7 @@ def time_candidates(plans: Sequence, bufs, shape: Tuple[int, int, int], stream=N
 def pick(plans_by_rank: Sequence[Tuple[int, object]], bufs, shape: Tuple[int, int, int], stream=None,
          margin: float = TIE_MARGIN) -> Tuple[int, List[Tuple[int, float]]]:
     """Times the candidates and applies ``choose``.  Returns ``(kept rank, [(rank, ms), ...])``."""
-    ms = time_candidates([p for _, p in plans_by_rank], bufs, shape, stream=stream)
+    ms = time_candidates([p for _, p in plans_by_rank], bufs, shape, stream=stream, settle_ms=PICK_SETTLE_MS)
     timings = [(rank, t) for (rank, _), t in zip(plans_by_rank, ms)]
     return choose(timings, margin), timings
 
