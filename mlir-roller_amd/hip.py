@@ -15,6 +15,7 @@ from __future__ import annotations
 import ctypes as C
 import os
 import subprocess
+import sys
 from dataclasses import dataclass, fields
 from pathlib import Path
 from typing import Optional, Sequence
@@ -632,7 +633,11 @@ def precompile_many(configs: Sequence[GemmConfig], jobs: Optional[int] = None) -
     cache_dir = _cache_dir_override or os.environ.get("ROLLER_HIP_CACHE", str(DEFAULT_CACHE_DIR))
     work = [(cache_dir, tuple(getattr(c, f.name) for f in fields(c))) for c in todo]
     failed = {}
-    if jobs <= 1 or len(todo) <= 1:
+    # a spawned worker re-imports the parent's main module by path; a parent that was fed from a pipe or
+    # typed at the prompt has none, and its workers would die on start
+    main_file = getattr(sys.modules.get("__main__"), "__file__", None)
+    spawnable = main_file is None or os.path.exists(main_file)
+    if jobs <= 1 or len(todo) <= 1 or not spawnable:
         results = list(map(_precompile_worker, work))
     else:
         with cf.ProcessPoolExecutor(max_workers=min(jobs, len(todo)), mp_context=mp.get_context("spawn")) as pool:
