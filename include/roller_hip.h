@@ -219,13 +219,15 @@ int rl_gemm_plan_launch(const rl_gemm_plan* plan, const float* A, const float* B
                         int M, int N, int K, int lda, int ldb, int ldc, rl_stream stream);
 
 /* Stream-K plans (cfg.streamk > 0) need a workspace: arrival counters (one unsigned per tile, zero
- * before a launch; the kernel leaves them at zero) followed by two slots of bm*bn floats per
- * workgroup.  rl_gemm_plan_launch takes it from the library, which keeps one per stream (allocated or
+ * before a launch; the kernel leaves them at zero; the area is 256 KiB for up to 65536 tiles and
+ * grows beyond) followed by two slots of bm*bn floats per workgroup.  rl_gemm_plan_launch takes it from the library, which keeps one per stream (allocated or
  * grown on first need, which synchronises that stream; launches on one stream run in order, and
  * launches on different streams use different workspaces).  rl_gemm_plan_launch_ws takes it from the
  * caller: `workspace` is device memory, 256-byte aligned, of at least rl_gemm_plan_workspace_bytes
- * bytes, whose first *counter_bytes bytes were zero before its first use; launches that share a
- * workspace must not overlap on the device.  For a plan without streamk both behave like
+ * bytes, whose first *counter_bytes bytes were zero before its first use -- and are zeroed again by
+ * the caller before a launch whose *counter_bytes is larger than that of the launches the workspace
+ * has served (only launches of more than 65536 tiles: their counters reach into what held the slots
+ * of the others); launches that share a workspace must not overlap on the device.  For a plan without streamk both behave like
  * rl_gemm_plan_launch and the workspace is ignored (bytes = 0).  No counterpart in the reference
  * (src/roller.py:545-550 launches one block per tile). */
 int rl_gemm_plan_workspace_bytes(const rl_gemm_plan* plan, int M, int N, int K, size_t* bytes, size_t* counter_bytes);

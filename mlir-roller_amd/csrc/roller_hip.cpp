@@ -443,9 +443,16 @@ int sk_make_params(const rl_gemm_config& c, int M, int N, int K, int compute_uni
   return RL_OK;
 }
 
-// Workspace of one stream-K launch: the arrival counters (one per tile, rounded up to 256 bytes),
-// then two slots of bm*bn floats per workgroup.
-size_t sk_counter_bytes(unsigned tiles) { return ((size_t)tiles * 4 + 255) / 256 * 256; }
+// Workspace of one stream-K launch: the arrival counters (one per tile; 256 KiB of them at least, so
+// that every launch of up to 65536 tiles keeps them in the same place, then rounded up to 256 bytes),
+// then two slots of bm*bn floats per workgroup.  The counter area must be zero when a launch starts
+// and is zero again when it ends; the slots may hold anything.  A workspace that is reused for a
+// launch with a LARGER counter area has pieces of earlier launches where the new counters go: whoever
+// owns the workspace zeroes the counter area again (the library does for its own, below).
+size_t sk_counter_bytes(unsigned tiles) {
+  const size_t need = ((size_t)tiles * 4 + 255) / 256 * 256;
+  return need > RL_STATIC_SCRATCH_COUNTER_BYTES ? need : (size_t)RL_STATIC_SCRATCH_COUNTER_BYTES;
+}
 size_t sk_workspace_bytes(const rl_gemm_config& c, const sk_params& p, unsigned tiles) {
   return sk_counter_bytes(tiles) + (size_t)2 * p.grid * c.bm * c.bn * 4;
 }
@@ -457,13 +464,22 @@ size_t sk_workspace_bytes(const rl_gemm_config& c, const sk_params& p, unsigned 
 struct Workspace {
   void* ptr = nullptr;
   size_t bytes = 0;
+  size_t counter_bytes = 0;   // the counter area the last launch used (zero from there to the front)
 };
 std::map<hipStream_t, Workspace> g_workspaces;
 std::mutex g_workspaces_mutex;   // (its own lock: launches hold the plan table's shared lock when they get here)
 
-int workspace_for(hipStream_t stream, size_t bytes, void** out) {
+int workspace_for(hipStream_t stream, size_t bytes, size_t counter_bytes, void** out) {
   std::lock_guard<std::mutex> lock(g_workspaces_mutex);
   Workspace& w = g_workspaces[stream];
+  if (w.bytes >= bytes && w.counter_bytes != counter_bytes) {
+    // the counter area moves its end (only launches of more than 65536 tiles differ): what lies between
+    // the two ends held slots of one launch and holds counters of the other.  Zeroed on the launch
+    // stream, behind the launches that used the old layout and ahead of the one that uses the new.
+    const size_t upto = w.counter_bytes > counter_bytes ? w.counter_bytes : counter_bytes;
+    HIP_TRY(hipMemsetAsync(w.ptr, 0, upto, stream));
+    w.counter_bytes = counter_bytes;
+  }
   if (w.bytes < bytes) {
     if (w.ptr) {
       // the old one may still be in use by a launch queued on this stream
@@ -477,6 +493,7 @@ int workspace_for(hipStream_t stream, size_t bytes, void** out) {
     // that does not synchronise with the default stream
     HIP_TRY(hipMemsetAsync(w.ptr, 0, want, stream));
     w.bytes = want;
+    w.counter_bytes = counter_bytes;
   }
   *out = w.ptr;
   return RL_OK;
@@ -553,7 +570,7 @@ int launch_plan(const rl_gemm_plan* plan, const float* A, const float* B, float*
     if ((uintptr_t)user_ws & 255) return fail(RL_ERR_INVALID_ARG, "workspace must be 256-byte aligned");
     ws = user_ws;
   } else {
-    rc = workspace_for((hipStream_t)stream, need, &ws);
+    rc = workspace_for((hipStream_t)stream, need, counter_room, &ws);
     if (rc) return rc;
   }
   unsigned* arrivals = (unsigned*)ws;

@@ -603,6 +603,9 @@ BEYOND_4GIB = [
     ("B", (256, 65792, 16384), GemmConfig(256, 256, 32, 128, 128, 32, 3, 0, 0, 4, 0, 3, 8, 0, 1)),
     ("C", (32768, 32900, 32), GemmConfig(256, 256, 32, 64, 128, 32, 3, 0, 0, 4, 1, 3, 8, 0, 1)),
     ("C-staged", (32768, 32900, 40), GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1)),
+    # the stream-K form: segments rebased to their first K step far into A; C beyond 4 GiB, every 130th tile split in two
+    ("A-streamk", (65792, 256, 16384), GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2)),
+    ("C-streamk", (32768, 33028, 96), GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 4, 2, 3, 8, 0, 1, 0, 2)),
 ]
 
 

@@ -174,6 +174,21 @@ def test_streamk_with_the_callers_workspace(device):
     assert np.array_equal(dC.get(), want)
 
 
+def test_a_launch_with_more_counters_behind_one_with_fewer_on_the_same_workspace(device):
+    """The library's workspace is reused from launch to launch.  A launch of more than 65536 tiles keeps
+    counters where an earlier launch kept the slots of its first workgroups; the library has to zero that
+    stretch again, or the tiles whose counters lie there never see their last piece arrive."""
+    small = GemmConfig(16, 16, 32, 16, 16, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2)      # 1 KiB slots right behind 256 KiB of counters
+    many = GemmConfig(32, 32, 32, 16, 16, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2)
+    first, second = (16, 16, 2048), (8224, 8256, 96)                               # 1 tile in 64 pieces; 66306 tiles, most shares end inside a tile
+    assert hip.streamk_schedule(many, *second, device.compute_units).counter_bytes > hip.streamk_schedule(small, *first, device.compute_units).counter_bytes == 256 * 1024
+    A1, B1 = go.make_inputs(*first, seed=5, distribution="integer")
+    A2, B2 = go.make_inputs(*second, seed=6, distribution="integer")
+    for _ in range(2):                                                                # and back again: the smaller layout behind the larger
+        assert np.array_equal(run(small, A1, B1), host_gemm(A1, B1))
+        assert np.array_equal(run(many, A2, B2), go.gemm_f32(A2, B2))
+
+
 def test_streamk_degenerate_extents(device):
     cfg = GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1, 0, 2)
     plan = GemmPlan(cfg)
