@@ -459,8 +459,8 @@ size_t sk_workspace_bytes(const rl_gemm_config& c, const sk_params& p, unsigned 
 
 // Workspaces the library owns, one per stream (launches on one stream run in order; launches on
 // different streams may overlap and must not share counters or slots).  Grown on demand, zeroed
-// when allocated (the kernels leave the counters at zero), freed never: a stream's last workspace
-// lives until the process ends.
+// when allocated (the kernels leave the counters at zero), freed with its stream (rl_stream_destroy);
+// the default stream's lives until the process ends.
 struct Workspace {
   void* ptr = nullptr;
   size_t bytes = 0;
@@ -768,6 +768,19 @@ int rl_stream_create(rl_stream* out) {
 int rl_stream_destroy(rl_stream s) {
   if (!s) return RL_OK;
   READY_OR_RETURN();
+  {
+    // the stream's stream-K workspace goes with it (a later stream may get the same handle value, and a
+    // process that makes and drops streams must not keep 64 MiB for each)
+    std::lock_guard<std::mutex> lock(g_workspaces_mutex);
+    auto it = g_workspaces.find((hipStream_t)s);
+    if (it != g_workspaces.end()) {
+      if (it->second.ptr) {
+        HIP_TRY(hipStreamSynchronize((hipStream_t)s));
+        HIP_TRY(hipFree(it->second.ptr));
+      }
+      g_workspaces.erase(it);
+    }
+  }
   HIP_TRY(hipStreamDestroy((hipStream_t)s));
   return RL_OK;
 }
