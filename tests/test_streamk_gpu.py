@@ -174,6 +174,32 @@ def test_streamk_with_the_callers_workspace(device):
     assert np.array_equal(dC.get(), want)
 
 
+def test_launches_back_to_back_share_the_library_workspace(device):
+    """The forty-eight seeded stream-K problems again, but all of them queued on one stream with no
+    synchronisation in between, forwards and then backwards: tile sizes, tile counts and grids change from
+    launch to launch, the library's workspace grows in the middle of the queue, and every launch has to find
+    the counters at zero and nobody else's pieces in its slots."""
+    sys.path.insert(0, str(__import__("pathlib").Path(__file__).resolve().parent))
+    from gemm_cases import seeded_streamk_cases
+    stream = hip.Stream()
+    cases = [(cfg, shape) for _, cfg, shape in seeded_streamk_cases() if not cfg.accum]
+    queued = []
+    for order in (cases, cases[::-1]):
+        for i, (cfg, (M, N, K)) in enumerate(order):
+            A, B = go.make_inputs(M, N, K, seed=4000 + i, distribution="integer")
+            dA, dB = DeviceArray.from_host(A), DeviceArray.from_host(B.T if cfg.trans_b else B)
+            dC = DeviceArray((M, N))
+            dC.fill_bytes(0xFF)
+            queued.append((cfg, (M, N, K), A, B, dA, dB, dC, GemmPlan(cfg)))
+    hip.synchronize()
+    for cfg, (M, N, K), _, _, dA, dB, dC, plan in queued:           # nothing but launches from here to the synchronisation
+        plan.launch(dA, dB, dC, M, N, K, stream=stream)
+    hip.synchronize()
+    assert len(queued) >= 60
+    for cfg, shape, A, B, _, _, dC, _ in queued:
+        assert np.array_equal(dC.get(), go.gemm_f32(A, B)), (cfg.tag(), shape)
+
+
 def test_a_launch_with_more_counters_behind_one_with_fewer_on_the_same_workspace(device):
     """The library's workspace is reused from launch to launch.  A launch of more than 65536 tiles keeps
     counters where an earlier launch kept the slots of its first workgroups; the library has to zero that
