@@ -75,7 +75,8 @@ typedef struct rl_gemm_config {
   int group;       /* panel height in tiles (reference: panel-width=8, roller.py:338)*/
   int accum;       /* 0: C = A*B, 1: C += A*B (linalg.matmul semantics, roller.py:62)*/
   int direct;      /* 1: global loads write LDS directly (no staging registers, swizzled
-                      A rows); needs stages>=3, vec=4, pad_a=pad_b=0, bk a power of 2 */
+                      A rows); needs stages>=3, pad_a=pad_b=0, bk a power of 2, and with
+                      vec=1 stages=3 and edge=1                                       */
   int trans_b;     /* 1: the second operand is Bt[N][ldb>=K], C = A*Bt^T (the [spatial, reduce]
                       layout of MatmulConfig.get_input_shapes, src/analyze.py:33-41); pad_b then
                       pads the K-contiguous rows of its LDS tile like pad_a                   */

@@ -114,11 +114,14 @@ def loads_go_direct_to_lds(matmul_config: "MatmulConfig", block_tile: Sequence[i
                            pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> bool:
     """Whether the MFMA kernel built for this tile uses its direct-to-LDS path (unpadded,
     XOR-swizzled rows; no staging registers): on the pipelined loop (pipeline depth 2 and up), with
-    128-bit global accesses (K and N multiples of 4), a power-of-two reduce step, and operand tiles
-    that are whole waves of 16-byte units.  The policy's LDS and register models and the mapping
-    from a hint to template parameters all ask this one function."""
+    a power-of-two reduce step and operand tiles that are whole waves of 16-byte units.  Rows that
+    are only dword-aligned (K or N not a multiple of 4) take it with two LDS buffers only (depths 2
+    and 3).  The policy's LDS and register models and the mapping from a hint to template parameters
+    all ask this one function."""
     m, n = block_tile
-    return (kernel_stages(pipeline_depth) >= 3 and matmul_config.K % 4 == 0 and matmul_config.N % 4 == 0
+    stages = kernel_stages(pipeline_depth)
+    aligned = matmul_config.K % 4 == 0 and matmul_config.N % 4 == 0
+    return (stages >= 3 and (aligned or stages == 3)
             and rstep & (rstep - 1) == 0 and (m * rstep // 4) % 64 == 0 and (rstep * n // 4) % 64 == 0)
 
 

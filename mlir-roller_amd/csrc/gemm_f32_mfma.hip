@@ -43,8 +43,13 @@
 //   GROUP, NXCD panel height in tiles; number of XCDs the dispatcher round-robins over
 //   ACCUM       1 = C += A*B (what linalg.matmul means, roller.py:62), 0 = C = A*B
 //   DIRECT      1 = global loads write LDS directly (buffer_load_dwordx4 ... lds), no staging
-//               registers and no LDS write instructions; needs STAGES>=3, VEC=4, PAD_A=PAD_B=0
-//               and BK a power of two.
+//               registers and no LDS write instructions; needs STAGES>=3, PAD_A=PAD_B=0
+//               and BK a power of two.  With VEC=1 (dword-aligned rows; STAGES=3 and EDGE=1
+//               then) full K steps are loaded the same way, at dword alignment, and the step
+//               that K ends in with buffer_load_dword ... lds, one float per lane and four
+//               instructions per 16-byte unit: every float is then inside its matrix or not on
+//               its own, where a 16-byte unit across the end of a row of A would bring the next
+//               row's first floats with it.
 //               A wave's load lands as 64 consecutive 16-byte units, so rows cannot be padded;
 //               instead the 16-byte chunks of every A row are XOR-swizzled with the row number
 //               (on the load side by choosing which global chunk a lane fetches, on the read
@@ -220,11 +225,19 @@ static_assert(STAGES >= 1 && STAGES <= 5, "pipeline depth 1 to 5");
 static_assert(STAGES <= 3 || DIRECT, "more than two LDS buffers only with direct-to-LDS loads");
 static_assert(VEC == 4 || VEC == 1, "global access width");
 static_assert(STREAMK >= 0 && (!STREAMK || STAGES == 3), "the stream-K variant is built on the pipelined loop with two LDS buffers");
-static_assert(!DIRECT || (STAGES >= 3 && VEC == 4 && PAD_A == 0 && PAD_B == 0), "DIRECT needs STAGES>=3, VEC=4, no padding");
+static_assert(!DIRECT || (STAGES >= 3 && PAD_A == 0 && PAD_B == 0), "DIRECT needs STAGES>=3 and no padding");
 /* Waiting for "all but the newest n tiles" counts this wave's outstanding loads, which is exact
  * only if every wave issues the same number of loads per tile. */
+// With dword-aligned rows (VEC == 1) the direct-to-LDS loads of a full K step are the same 16-byte
+// units per lane (the memory pipeline accepts dword alignment for them), but a unit that straddles
+// the end of K would bring the next row's first floats with it: the steps that may hold the end of K
+// load one float per lane instead, four instructions for every one, each float tested by itself.
+#define DW_DIRECT (DIRECT && VEC == 1)
 #define LOADS_PER_TILE (A_PER_T + B_PER_T)
+#define A_DW_LOADS ((4 * A_UNITS + NT - 1) / NT)
+#define B_DW_LOADS ((4 * B_UNITS + NT - 1) / NT)
 #define EXACT_LOADS (A_UNITS % NT == 0 && B_UNITS % NT == 0)
+static_assert(!DW_DIRECT || (LDS_BUFS == 2 && EDGE == 1), "direct-to-LDS loads of dword-aligned rows: two LDS buffers, all three extents tested");
 static_assert(LDS_BUFS <= 2 || EXACT_LOADS, "three or more LDS buffers need operand tiles that divide evenly over the threads");
 static_assert(LDS_BUFS <= 2 || (LDS_BUFS - 2) * LOADS_PER_TILE <= 63, "too many loads in flight for the 6-bit vmcnt");
 /* the prologue may start on tile 0 while the other requested tiles are still in flight, if that
@@ -539,7 +552,8 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 
 #if DIRECT
   // Issues the loads of K step kt straight into LDS buffer `stage`.  Instruction i of a wave
-  // fills the 64 consecutive 16-byte units that start at unit i*NT + wave*64 of the operand tile.
+  // fills the 64 consecutive 16-byte units (floats, with dword-aligned rows) that start at unit
+  // i*NT + wave*64 of the operand tile.
   // KTAIL (a compile-time 0/1) says whether tile kt may be the one that K ends in: only then are
   // the units tested against K.
   auto fetch_direct = [&](auto ktail, int kt, int stage) __attribute__((always_inline)) {
@@ -551,19 +565,62 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const __amdgpu_buffer_rsrc_t br = tile_rsrc(Bg + B_STEP(k0), live, b_rem - B_STEP(k0) * 4);
     float* As = lds + stage * A_STAGE;
     float* Bs = lds + LDS_BUFS * A_STAGE + stage * B_STAGE;
+    if constexpr (DW_DIRECT && KTEST) {
+      // Dword-aligned rows.  A tile past the end needs no request (no wait of this variant counts
+      // loads: two LDS buffers), a full tile takes the 16-byte loads below, and the tile that K ends
+      // in is loaded one float per lane: instruction j of a wave fills the 64 consecutive floats that
+      // start at float j*NT + wave*64 of the operand tile's LDS image; float d of the image is
+      // element d % 4 of 16-byte unit d / 4.  That is once per tile, so the offsets are worked out
+      // from the thread number here (behind an opaque copy: otherwise they would be hoisted and
+      // kept in registers across the loop) rather than carried.
+      if (!live) return;
+    }
+    if (DW_DIRECT && KTEST && k0 + BK > Kl) {
+      int t = tid;
+      asm volatile("" : "+v"(t));
+#pragma unroll
+      for (int j = 0; j < A_DW_LOADS; ++j) {
+        const int first = j * NT + wave * 64;
+        if ((4 * A_UNITS) % NT == 0 || first < 4 * A_UNITS) {
+          const int d = t + j * NT, u = d / 4, row = u / CPR, k = ((u % CPR) ^ ((row / RPL) % SWZ_N)) * 4 + d % 4;
+          const bool ok = m0 + row < M && k0 + k < Kl;
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr_t)(As + first), 4, ok ? (unsigned)(row * lda + k) * 4u : OOB_OFFSET, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < B_DW_LOADS; ++j) {
+        const int first = j * NT + wave * 64;
+        if ((4 * B_UNITS) % NT == 0 || first < 4 * B_UNITS) {
+          const int d = t + j * NT, u = d / 4;
+#if TRANS_B
+          const int row = u / CPR, k = ((u % CPR) ^ ((row / RPL) % SWZ_N)) * 4 + d % 4, col = bt_col_of_row(row);
+          const bool ok = n0 + col < N && k0 + k < Kl;
+          const unsigned off = (unsigned)(col * ldb + k) * 4u;
+#else
+          const int krow = u / (BN / 4), col = b_tile_col(krow, u % (BN / 4) * 4) + d % 4;
+          const bool ok = n0 + col < N && k0 + krow < Kl;
+          const unsigned off = (unsigned)(krow * ldb + col) * 4u;
+#endif
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(br, (lds_ptr_t)(Bs + first), 4, ok ? off : OOB_OFFSET, 0, 0, 0);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < A_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (A_UNITS % NT == 0 || first < A_UNITS) {
-        const bool ok = a_ok[i] && (!KTEST || k0 + a_kcol[i] < Kl);
+        const bool ok = a_ok[i] && (!KTEST || DW_DIRECT || k0 + a_kcol[i] < Kl);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ar, (lds_ptr_t)(As + first * 4), 16, ok ? a_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
+    // (B[K,N] with dword-aligned rows: a unit that straddles N is loaded if its first column is inside;
+    // what it brings beyond N only ever meets columns of C that are not stored)
 #pragma unroll
     for (int i = 0; i < B_PER_T; ++i) {
       const int first = i * NT + wave * 64;
       if (B_UNITS % NT == 0 || first < B_UNITS) {
-        const bool ok = b_ok[i][0] && (!KTEST || k0 + b_krow[i] < Kl);  // K % 4 == 0: a chunk is in or out as a whole
+        const bool ok = b_ok[i][0] && (!KTEST || DW_DIRECT || k0 + b_krow[i] < Kl);  // K % 4 == 0: a chunk is in or out as a whole
         __builtin_amdgcn_raw_ptr_buffer_load_lds(br, (lds_ptr_t)(Bs + first * 4), 16, ok ? b_goff[i] : OOB_OFFSET, 0, 0, 0);
       }
     }
@@ -719,10 +776,17 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     const int pipelined = KT - 1;
     const int first = pipelined & 1;
 #if DIRECT
+    // (dword-aligned rows: the number of loads per tile is known only if K cannot end in these tiles)
+    if (!DW_DIRECT || KT > LDS_BUFS) {
 #pragma unroll
-    for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(int_c<1>{}, i, LDS_BUFS == 2 ? (i ^ first) : i);
-    // this wave's part of tile 0 is in LDS (of every requested tile when the loads per wave differ)
-    WAIT_VMCNT(PROLOGUE_IN_FLIGHT);
+      for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(int_c<!DW_DIRECT>{}, i, LDS_BUFS == 2 ? (i ^ first) : i);
+      // this wave's part of tile 0 is in LDS (of every requested tile when the loads per wave differ)
+      WAIT_VMCNT(PROLOGUE_IN_FLIGHT);
+    } else {
+#pragma unroll
+      for (int i = 0; i < LDS_BUFS; ++i) fetch_direct(int_c<1>{}, i, LDS_BUFS == 2 ? (i ^ first) : i);
+      WAIT_VMCNT(0);
+    }
 #else
     fetch(int_c<1>{}, 0);
     stash(first);
@@ -738,11 +802,12 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // P = which of the two fragment sets holds round 0 of this step (compile-time, so that the
     // sets stay in fixed registers); the set alternates every round.
     // MFMAs and fragment reads per round; LDS writes and global loads per K step
-    constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NSEG), W = A_PER_T + B_PER_T, L = W * (VEC == 4 ? 1 : 4);
+    constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NSEG), W = A_PER_T + B_PER_T, L0 = DIRECT ? LOADS_PER_TILE : W * (VEC == 4 ? 1 : 4);
 
     // `buffer`: the LDS buffer of this step's tile when there are two (with more, kt % LDS_BUFS).
     auto step = [&](auto parity, auto ktail, auto buffer, int kt) __attribute__((always_inline)) {
       constexpr int P = decltype(parity)::value;
+      constexpr int L = L0;
       const int cur = LDS_BUFS == 2 ? decltype(buffer)::value : (unsigned)kt % LDS_BUFS;
       const int nxt = LDS_BUFS == 2 ? 1 - decltype(buffer)::value : (unsigned)(kt + 1) % LDS_BUFS;
 #pragma unroll
@@ -897,6 +962,15 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   // with fences the split cost more than it saved).  A writer waits until its stores have been
   // acknowledged (vmcnt 0) before its workgroup is counted in; the reader only reads once it has
   // seen the count.
+  //
+  // Everything below that depends on the thread number alone is the same for every segment, and
+  // the compiler would work it out once, ahead of the segment loop, and keep it in registers through
+  // every K loop (40 to 90 of them: the difference between one and two workgroups per CU for the
+  // larger tiles).  The epilogue therefore derives its lane coordinates from an opaque copy.
+  int tid_here = threadIdx.y * blockDim.x + threadIdx.x;
+  asm volatile("" : "+v"(tid_here));
+  const int tid = tid_here, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / NWN) * WM, wn0 = (wave % NWN) * WN, lr = lane % MI, lg = lane / MI;
   bool store_c = true;
   if (seg.kb != 0 || seg.ke != sk.kt) {
     constexpr int CHUNKS = ACC_REGS / 4;            // 16-byte chunks per MFMA block and lane

@@ -149,8 +149,10 @@ int check_config(const rl_gemm_config& c, int* lds_bytes, int* threads) {
   if ((c.swz & 2) && c.group <= 0) return fail(RL_ERR_INVALID_ARG, "group must be positive");
   if ((c.direct | 1) != 1) return fail(RL_ERR_INVALID_ARG, "direct is 0 or 1");
   if (c.direct) {
-    if (c.stages < 3 || c.vec != 4 || c.pad_a || c.pad_b)
-      return fail(RL_ERR_INVALID_ARG, "direct=1 needs stages>=3, vec=4, pad_a=0, pad_b=0");
+    if (c.stages < 3 || c.pad_a || c.pad_b)
+      return fail(RL_ERR_INVALID_ARG, "direct=1 needs stages>=3, pad_a=0, pad_b=0");
+    if (c.vec == 1 && (c.stages != 3 || c.edge != 1))
+      return fail(RL_ERR_INVALID_ARG, "direct=1 with vec=1 (dword-aligned rows) needs stages=3 and edge=1, got stages=%d edge=%d", c.stages, c.edge);
     if (c.bk & (c.bk - 1)) return fail(RL_ERR_INVALID_ARG, "direct=1 needs bk to be a power of two (XOR swizzle), got %d", c.bk);
     if ((c.bm * c.bk / 4) % 64 || (c.bk * c.bn / 4) % 64)
       return fail(RL_ERR_INVALID_ARG, "direct=1 needs bm*bk and bk*bn to be multiples of 256 (whole waves of 16-byte units)");

@@ -43,8 +43,9 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
     block_tile -> BM, BN; rstep -> BK; wave_tile -> WM, WN (derived from the thread count when
     the hint comes from a device model without matrix cores); pipeline_depth -> pipeline stages
     (``kernel_stages``: the reference's depth 2 and the sweep's depth 3 are the same kernel, two LDS
-    buffers and the pipelined loop; 4 and 5 add buffers).  Ragged problems switch on predication, and problems whose K, N
-    are not multiples of 4 fall back to dword global accesses.  ``trans_b`` selects the kernel
+    buffers and the pipelined loop; 4 and 5 add buffers).  Ragged problems switch on predication, and
+    problems whose K, N are not multiples of 4 get the kernel for dword-aligned rows (vec=1; it keeps
+    the direct-to-LDS loads with two LDS buffers).  ``trans_b`` selects the kernel
     whose second operand is stored as Bt[N, K].
     """
     bm, bn = hint.block_tile
@@ -76,7 +77,7 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
                 and (stages - 1) * (bm * bk + bk * bn) * 4 <= MI355X().lds_bytes):
             break
         stages -= 1
-    # At full depth and width the global loads go straight to LDS (swizzled A rows, no padding)
+    # On the pipelined loop the global loads go straight to LDS (swizzled A rows, no padding)
     # whenever both operand tiles are whole waves of 16-byte units and the K step is a power of
     # two (the swizzle is an XOR).
     direct = int(loads_go_direct_to_lds(config, (bm, bn), bk, stages))
@@ -96,7 +97,8 @@ def hint_to_gemm_config(config: MatmulConfig, hint: TileDict, pipeline_depth: in
     return GemmConfig(
         bm=bm, bn=bn, bk=bk, wm=wm, wn=wn, mi=mi, stages=stages, pad_a=pad_a, pad_b=pad_b, vec=vec,
         # 0: every extent is a whole number of tiles; 2: only M or N is ragged; 1: K is ragged too
-        edge=(0 if (M % bm == 0 and N % bn == 0) else 2) if K % bk == 0 else 1,
+        # (the direct-to-LDS loads of dword-aligned rows come with all three tests)
+        edge=(0 if (M % bm == 0 and N % bn == 0) else 2) if K % bk == 0 and not (direct and vec == 1) else 1,
         swz=3, group=8, accum=1 if accumulate else 0, direct=direct, trans_b=1 if trans_b else 0,
         # the stream-K form of the kernel exists on the pipelined loop only
         streamk=int(getattr(hint, "stream_k", 0)) if stages == 3 else 0,

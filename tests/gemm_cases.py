@@ -117,3 +117,34 @@ def seeded_streamk_cases(count: int = 48, seed: int = STREAMK_SEED):
         yield case, sk, (M, N, K)
         case += 1
 
+
+
+DWORD_DIRECT_SEED = 20251125
+
+
+def seeded_dword_direct_cases(count: int = 40, seed: int = DWORD_DIRECT_SEED):
+    """Yields ``(case, GemmConfig, (M, N, K))``: the draw of ``seeded_template_cases`` (another seed)
+    moved onto the direct-to-LDS loads of dword-aligned rows -- vec=1 with direct=1, which means the
+    pipelined loop on two buffers, all three extents tested, no padding -- a third of them as stream-K.
+    N and K are drawn again, odd ones included; K runs from less than one K step (the tile K ends in
+    is the first) over exactly two (no tile is cut short) to a dozen.  Only configurations that
+    ``rl_gemm_config_check`` accepts are kept."""
+    import dataclasses
+
+    from mlir_roller_amd import hip
+
+    rng = np.random.default_rng(seed + 1)
+    case = 0
+    for _, cfg, (M, _, _) in seeded_template_cases(count=6 * count, seed=seed):
+        if case == count:
+            break
+        dw = dataclasses.replace(cfg, vec=1, direct=1, stages=3, edge=1, pad_a=0, pad_b=0,
+                                 streamk=int(rng.choice([0, 0, 1, 2])))
+        N = int(rng.integers(1, 3 * cfg.bn))
+        K = int(rng.choice([rng.integers(1, cfg.bk + 1), 2 * cfg.bk, 3 * cfg.bk - 1, rng.integers(1, 12 * cfg.bk)]))
+        try:
+            hip.config_check(dw)
+        except hip.HipError:
+            continue
+        yield case, dw, (M, N, K)
+        case += 1

@@ -85,7 +85,8 @@ def test_config_check_accepts_and_sizes(hip_lib):
     (dict(accum=2), "accum is 0 or 1"),
     (dict(mi=16, bk=8), "bk must be a multiple of 16"),
     (dict(direct=1), "direct=1 needs stages>=3"),
-    (dict(direct=1, stages=3, pad_a=0, vec=1), "direct=1 needs stages>=3"),
+    (dict(direct=1, stages=3, pad_a=0, vec=1, edge=2), "direct=1 with vec=1 (dword-aligned rows) needs stages=3 and edge=1"),
+    (dict(direct=1, stages=4, pad_a=0, vec=1, edge=1, bk=32), "direct=1 with vec=1 (dword-aligned rows) needs stages=3 and edge=1"),
     (dict(direct=2), "direct is 0 or 1"),
     (dict(direct=1, stages=3, pad_a=0, bk=24), "power of two"),
 ])

@@ -293,6 +293,27 @@ def test_seeded_points_of_the_template_parameter_space_are_exact(device):
     assert len(seen) >= 60          # the draw really spreads over the parameter space
 
 
+def test_direct_to_lds_loads_of_dword_aligned_rows_are_exact(device):
+    """Forty seeded (configuration, shape) pairs on the direct-to-LDS path with dword-aligned rows
+    (any N and K; full K steps come with 16-byte loads at dword alignment, the step K ends in one
+    float per lane), a third of them as stream-K: integer inputs, bit-exact against the oracle, each
+    at its drawn K and with one K step more."""
+    from gemm_cases import seeded_dword_direct_cases
+    tails = set()
+    for case, cfg, (M, N, K0) in seeded_dword_direct_cases():
+        for K in (K0, K0 + cfg.bk):
+            say("dword-aligned direct case", case, cfg.tag(), (M, N, K))
+            A, B = go.make_inputs(M, N, K, seed=3000 + case, distribution="integer")
+            want = go.gemm_f32(A, B)
+            if cfg.accum:
+                C0 = np.random.default_rng(case).integers(0, 10, (M, N)).astype(np.float32)
+                assert np.array_equal(run_gemm(cfg, A, B, c_init=C0), want + C0), (case, cfg.tag(), K)
+            else:
+                assert np.array_equal(run_gemm(cfg, A, B), want), (case, cfg.tag(), K)
+        tails.add((K0 % cfg.bk == 0, -(-K0 // cfg.bk) <= 2, N % 4 == 0))
+    assert len(tails) >= 6          # whole and cut last steps, short and long K, N aligned or not
+
+
 def test_accumulate_mode_adds_into_c(device):
     M, N, K = 300, 260, 100
     A, B = go.make_inputs(M, N, K, seed=11, distribution="integer")

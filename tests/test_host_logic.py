@@ -46,8 +46,15 @@ def test_hint_to_gemm_config_ragged_problem():
     g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0])
     assert g.edge == 2 and g.vec == 4 and 1536 % g.bk == 0   # 5000 and 1536 are multiples of 4; K is a whole number of steps
     cfg = MatmulConfig(37, 53, 29, 32)
-    g = roller.hint_to_gemm_config(cfg, get_roller_hints(cfg, MI355X(), 1)[0], pipeline_depth=3)
-    assert g.edge == 1 and g.vec == 1 and g.direct == 0 and (g.mi, g.pad_a) == (16, 8)   # dword path keeps padded rows
+    hint = get_roller_hints(cfg, MI355X(), 1)[0]
+    g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=3)
+    assert (g.edge, g.vec, g.direct, g.stages, g.pad_a) == (1, 1, 1, 3, 0)    # dword-aligned rows still go straight to LDS ...
+    g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=5)
+    assert (g.edge, g.vec, g.direct, g.stages) == (1, 1, 1, 3)               # ... on two LDS buffers, whatever depth is asked for,
+    g = roller.hint_to_gemm_config(MatmulConfig(37, 53, 64, 32), hint, pipeline_depth=2)
+    assert (g.edge, g.vec, g.direct) == (1, 1, 1)                            # with all three extents tested (53 is odd, 64 a whole step)
+    g = roller.hint_to_gemm_config(cfg, hint, pipeline_depth=1)
+    assert (g.vec, g.direct, g.stages) == (1, 0, 1) and (g.mi, g.pad_a) == (16, 8)   # the unpipelined loop stages through registers: padded rows
 
 
 def test_hint_from_the_a100_model_still_maps_to_wave_tiles():

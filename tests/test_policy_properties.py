@@ -42,6 +42,7 @@ def test_every_mi355x_hint_is_a_valid_kernel_configuration(hip_lib, M, N, K):
         g = hint_to_gemm_config(cfg, h, 3)
         lds, threads = hip.config_check(g)              # the C ABI's own validation
         assert threads == h.threads and lds <= arch.lds_bytes
-        assert g.edge == (1 if K % g.bk else (2 if (M % g.bm or N % g.bn) else 0))   # K ragged / only M, N ragged / aligned
+        # K ragged (or dword-aligned rows loaded straight into LDS: always all three tests) / only M, N ragged / aligned
+        assert g.edge == (1 if K % g.bk or (g.direct and g.vec == 1) else (2 if (M % g.bm or N % g.bn) else 0))
         assert g.vec == (4 if K % 4 == 0 and N % 4 == 0 else 1)
         assert h.grid_size == math.ceil(M / g.bm) * math.ceil(N / g.bn)
