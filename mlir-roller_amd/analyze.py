@@ -296,6 +296,9 @@ class Policy:
     # registers per lane the MFMA kernel needs besides its accumulators and operand fragments:
     # addresses, loop state, buffer resources (measured: 40-60)
     REG_OVERHEAD = 50
+    # ... and what the kernel for dword-aligned rows (K or N not a multiple of 4) needs on top:
+    # exact buffer ranges, three extents of predicates (measured: 40 on whole tiles, 60 as stream-K)
+    DWORD_ROWS_REGS = 60
 
     def __init__(self, config: MatmulConfig, arch: TileDevice,
                  pipeline_depth: int = DEFAULT_PIPELINE_DEPTH) -> None:
@@ -453,6 +456,18 @@ class Policy:
         if self.estimate_seconds(td, workgroups) < self.estimate_seconds(td, 0) * (1.0 - a.stream_k_margin):
             td.stream_k = workgroups
 
+    def _stream_k_fit(self, hint: TileDict, workgroups: int) -> int:
+        """``workgroups`` per core of a stream-K kernel, cut down to what the register file holds once
+        the wave tile is known (a stream-K grid of more workgroups than are resident runs in rounds
+        again, with more pieces to add up)."""
+        arch = self.arch
+        if not workgroups or not hint.wave_tile or not arch.regs_per_lane:
+            return workgroups
+        acc_regs = int(math.prod(hint.wave_tile) // arch.warp_size * self.matmul_config.el_bytes / 4)
+        regs = acc_regs + self._reg_overhead(hint, hint.wave_tile, hint.mfma, hint.threads)
+        waves_per_simd = max(1, -(-(hint.threads // arch.warp_size) // arch.sm_partition))
+        return max(1, min(workgroups, arch.regs_per_lane // (waves_per_simd * regs)))
+
     def get_block_tiles_candidates(self, init_tile: List[int], rstep: int) -> List[TileDict]:
         """All valid block tiles, best first (stable with respect to enumeration order:
         m outer, n inner, ascending)."""
@@ -567,6 +582,8 @@ class Policy:
         it also stages one K step of both operand tiles in registers."""
         blocks_m, blocks_n = wave_tile[0] // mi, wave_tile[1] // mi
         regs = self.REG_OVERHEAD + 2 * 4 * (blocks_m + blocks_n)
+        if self.matmul_config.K % 4 or self.matmul_config.N % 4:
+            regs += self.DWORD_ROWS_REGS
         if not loads_go_direct_to_lds(self.matmul_config, td.block_tile, td.rstep, self.pipeline_depth):
             regs += -(-(sum(td.block_tile) * td.rstep) // block_size)
         return regs
@@ -632,9 +649,10 @@ class Policy:
         for td in self.get_block_tiles_candidates([1, 1], rstep):
             self._expand_reduce_axis(td)
             for hint in self.assign_thread_tile(td, 1 if mfma else 2):
+                hint.stream_k = self._stream_k_fit(hint, hint.stream_k)
                 hints.append(hint)
                 if mfma and self.arch.stream_k_workgroups and 2 <= self.pipeline_depth <= 3:
-                    other = max(1, min(self.arch.stream_k_workgroups, hint.block_per_SM)) if not hint.stream_k else 0
+                    other = self._stream_k_fit(hint, max(1, min(self.arch.stream_k_workgroups, hint.block_per_SM))) if not hint.stream_k else 0
                     mine, its = self.estimate_seconds(hint), self.estimate_seconds(hint, other)
                     if its < mine * (1.0 + self.STREAM_K_TOSS_UP) and len(hints) < topk:
                         twin = hint.clone()

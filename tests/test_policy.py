@@ -357,7 +357,8 @@ def test_mi355x_top_hints_compile_without_spills_or_scratch():
     from mlir_roller_amd import hip
     from mlir_roller_amd.benchmark import README_SHAPES
     seen = {}
-    for shape in list(README_SHAPES) + [(3000, 5000, 1536), (200, 300, 72), (2560, 2560, 2560), (1920, 2880, 2048)]:
+    for shape in list(README_SHAPES) + [(3000, 5000, 1536), (200, 300, 72), (2560, 2560, 2560), (1920, 2880, 2048),
+                                        (4095, 4097, 4093), (2049, 2047, 2051)]:
         cfg = MatmulConfig(*shape, 32)
         for h in get_roller_hints(cfg, MI355X(), topk=8):
             seen.setdefault(hint_to_gemm_config(cfg, h, 3), (shape, h))
@@ -369,8 +370,13 @@ def test_mi355x_top_hints_compile_without_spills_or_scratch():
         # of kernel get there, and within bounds: the one-wave tiles of tiny ragged problems (dozens of
         # per-load predicates) and the stream-K kernels (the split's parameters stay live across the
         # segments of a workgroup; their K loop itself carries no such traffic, which a GPU timing shows)
-        assert res["sgpr_spills"] == 0 or (res["sgpr_spills"] <= 64 and (g.threads == 64 or g.streamk)), (shape, g.tag(), res)
+        # -- and the kernels for dword-aligned rows (the step that K ends in works its offsets out again)
+        assert res["sgpr_spills"] == 0 or (res["sgpr_spills"] <= 64 and (g.threads == 64 or g.streamk)) \
+            or (res["sgpr_spills"] <= 128 and g.vec == 1), (shape, g.tag(), res)
         assert 0 < res["vgprs"] <= 512 // max(1, g.threads // 256), (g.tag(), res)
+        # a stream-K grid is sized for that many workgroups per CU: they have to fit the register file together
+        if g.streamk and g.threads >= 256:
+            assert res["vgprs"] <= 512 // (g.streamk * (g.threads // 256)), (shape, g.tag(), res)
 
 
 def test_mi355x_small_wave_tiles_list_the_long_k_instruction_first():
