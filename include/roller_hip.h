@@ -94,6 +94,8 @@ typedef struct rl_streamk_schedule {
   int tiles, tile_rows, tile_cols;
   long units;           /* tiles * k_steps; every workgroup gets units / grid of them, give or take one */
   size_t workspace_bytes, counter_bytes;
+  int whole_tiles;      /* a multiple of grid: the first so many tiles (in walk order) are worked whole,
+                           tile round * grid + g by workgroup g, after its share of the units of the rest */
 } rl_streamk_schedule;
 
 /* One run of K steps of one tile, as a workgroup of a stream-K launch works it. */

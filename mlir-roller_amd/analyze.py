@@ -435,13 +435,24 @@ class Policy:
         return tiles_per_cu * max(t_mfma, t_mem) + (-(-tiles_per_cu // resident)) * t_fixed
 
     def stream_k_pieces(self, td: TileDict, stream_k: int) -> float:
-        """How many workgroups meet in one tile of a stream-K launch: with fewer reduce steps in a
-        share than in a tile, a tile's steps / a share's steps, plus one for the share that straddles
-        its start; otherwise two (a share ends inside at most one tile).  The workgroup that arrives last
-        reads that many pieces of the tile back, one after the other, which is what a split costs."""
+        """How many workgroups meet in one split tile of a stream-K launch.  From two tiles per workgroup
+        on, all rounds of the grid but the last are worked as whole tiles (all of them, if the tile count
+        is a multiple of the grid: nothing is split then) and the reduce steps of the remaining tiles are
+        shared out: a share is at least a tile long and ends inside at most one tile, two pieces.  With
+        fewer tiles everything is shared out, and with fewer reduce steps in a share than in a tile a
+        tile has its steps / a share's steps pieces, plus one for the share that straddles its start.
+        The workgroup that arrives last reads that many pieces of the tile back, one after the other,
+        which is what a split costs."""
         k_steps = -(-self.matmul_config.K // td.rstep)
-        units = td.grid_size * k_steps
-        share = units / min(stream_k * self.arch.compute_max_core, units)
+        tiles = td.grid_size
+        grid = min(stream_k * self.arch.compute_max_core, tiles * k_steps)
+        rounds = tiles // grid - 1 if tiles >= 2 * grid else 0
+        if tiles >= grid and tiles % grid == 0:
+            rounds = tiles // grid
+        units = (tiles - rounds * grid) * k_steps
+        if not units:
+            return 0.0
+        share = units / grid
         return k_steps / share + 1.0 if share < k_steps else 2.0
 
     def _choose_stream_k(self, td: TileDict) -> None:
@@ -613,9 +624,14 @@ class Policy:
             acc_regs = int(math.prod(thread_tile) * self.matmul_config.el_bytes / 4)
             if acc_regs >= arch.thread_reg_limit:
                 continue
-            if budget and acc_regs + self._reg_overhead(td, wave_tile, mi, block_size) > budget:
+            regs = acc_regs + self._reg_overhead(td, wave_tile, mi, block_size)
+            if budget and regs > budget:
                 continue
             done = td.clone()
+            if budget and 2 * regs > budget and done.block_per_SM > 1:
+                # more than half of the registers its waves can have: the workgroup runs alone on its core
+                done.block_per_SM = 1
+                done.num_wave = -(-done.grid_size // arch.compute_max_core)
             done.thread_tile = thread_tile
             done.wave_tile = wave_tile
             done.mfma = mi

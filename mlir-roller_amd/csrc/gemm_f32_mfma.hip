@@ -443,13 +443,15 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   const int lg = lane / MI;  // k group inside an MFMA
 
 #if STREAMK
-  // This workgroup's share of the (tile, K step) units, one segment (a run of K steps of one tile) at
-  // a time.  All of it is wave-uniform scalar arithmetic.
+  // This workgroup's work, one segment (a run of K steps of one tile) at a time: first its share of
+  // the (tile, K step) units of the tiles that are shared out, then its whole tiles, one per round of
+  // the grid.  All of it is wave-uniform scalar arithmetic.
   unsigned wg = blockIdx.x;
   if (wg >= sk.grid) return;
 #if SWZ & 1
   {
     // workgroups are dealt to the XCDs round-robin: give every XCD one contiguous stretch of the units
+    // (and of the tiles of every round)
     const unsigned per = (sk.grid + NXCD - 1) / NXCD;
     unsigned tall = sk.grid % NXCD;
     if (tall == 0) tall = NXCD;
@@ -459,9 +461,16 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 #endif
   unsigned sk_unit = sk_first_unit(sk, wg);
   const unsigned sk_end = sk_first_unit(sk, wg + 1);
-  for (bool again = false; sk_unit < sk_end; again = true) {
-  const sk_segment seg = sk_segment_at(sk, sk_unit, sk_end);
-  sk_unit += seg.ke - seg.kb;
+  unsigned sk_tile = wg;                             // the next whole tile: wg, wg + grid, ... below dp_tiles
+  for (bool again = false; sk_unit < sk_end || sk_tile < sk.dp_tiles; again = true) {
+  sk_segment seg;
+  if (sk_unit < sk_end) {
+    seg = sk_segment_at(sk, sk_unit, sk_end);
+    sk_unit += seg.ke - seg.kb;
+  } else {
+    seg = sk_whole_tile(sk, sk_tile);
+    sk_tile += sk.grid;
+  }
   const int tile_m = (int)seg.tile_m, tile_n = (int)seg.tile_n;
   const int kb = (int)seg.kb;                       // first K step of the segment
   if (again) __syncthreads();                       // every wave is done with the LDS tiles of the previous segment
@@ -974,7 +983,7 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
   bool store_c = true;
   if (seg.kb != 0 || seg.ke != sk.kt) {
     constexpr int CHUNKS = ACC_REGS / 4;            // 16-byte chunks per MFMA block and lane
-    const unsigned tile_unit = seg.tile * sk.kt;     // unit number of the tile's first K step
+    const unsigned tile_unit = sk_tile_unit(sk, seg.tile);   // (shared) unit number of the tile's first K step
     const unsigned first_wg = sk_owner(sk, tile_unit);
     const unsigned pieces = sk_owner(sk, tile_unit + sk.kt - 1) - first_wg + 1;
     const unsigned my_slot = 2 * wg + (seg.kb == 0 ? 1 : 0);

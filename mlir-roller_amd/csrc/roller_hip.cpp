@@ -421,7 +421,9 @@ sk_div make_div(unsigned d) {
 
 // Fills *p for cfg on an M x N x K problem with `compute_units` CUs.  The grid is cfg.streamk
 // workgroups per CU, cut down to one K step per workgroup where the problem is smaller than that
-// (the decoding relies on no share being empty).
+// (the decoding relies on no share being empty, unless all are).  From two tiles per workgroup on,
+// all rounds of whole tiles but the last are worked as whole tiles (all of them if the tile count is
+// a multiple of the grid) and only the units of the remaining tiles are shared out.
 int sk_make_params(const rl_gemm_config& c, int M, int N, int K, int compute_units, sk_params* p, unsigned* tiles) {
   if (!c.streamk) return fail(RL_ERR_INVALID_ARG, "not a stream-K configuration");
   if (M <= 0 || N <= 0 || K <= 0) return fail(RL_ERR_INVALID_ARG, "stream-K needs M, N, K > 0 (M=%d N=%d K=%d)", M, N, K);
@@ -433,8 +435,13 @@ int sk_make_params(const rl_gemm_config& c, int M, int N, int K, int compute_uni
     return fail(RL_ERR_INVALID_ARG, "problem too large for the 32-bit arithmetic of the stream-K split (%lu units)", units);
   unsigned long grid = (unsigned long)compute_units * c.streamk;
   if (grid > units) grid = units;
+  const unsigned long n_tiles = nbm * nbn;
+  unsigned long rounds = n_tiles >= 2 * grid ? n_tiles / grid - 1 : 0;
+  if (n_tiles >= grid && n_tiles % grid == 0) rounds = n_tiles / grid;
+  const unsigned long shared = (n_tiles - rounds * grid) * kt;   // units that are shared out
   memset(p, 0, sizeof *p);
-  p->grid = (unsigned)grid; p->q = (unsigned)(units / grid); p->r = (unsigned)(units % grid); p->kt = (unsigned)kt;
+  p->grid = (unsigned)grid; p->dp_tiles = (unsigned)(rounds * grid);
+  p->q = (unsigned)(shared / grid); p->r = (unsigned)(shared % grid); p->kt = (unsigned)kt;
   p->nbm = (unsigned)nbm; p->nbn = (unsigned)nbn;
   p->group = (c.swz & 2) ? (unsigned)(c.group > 0 ? c.group : 1) : 1u;
   p->rows_last = (unsigned)(nbm % p->group);
@@ -1031,7 +1038,8 @@ int rl_gemm_streamk_schedule(const rl_gemm_config* cfg, int M, int N, int K, int
   out->tiles = (int)tiles;
   out->tile_rows = (int)sp.nbm;
   out->tile_cols = (int)sp.nbn;
-  out->units = (long)sp.grid * sp.q + sp.r;
+  out->units = (long)tiles * sp.kt;
+  out->whole_tiles = (int)sp.dp_tiles;
   out->workspace_bytes = sk_workspace_bytes(*cfg, sp, tiles);
   out->counter_bytes = sk_counter_bytes(tiles);
   return RL_OK;
@@ -1050,19 +1058,26 @@ int rl_gemm_streamk_segments(const rl_gemm_config* cfg, int M, int N, int K, int
   // exactly what a workgroup of the kernel does with its (logical) index
   unsigned unit = sk_first_unit(sp, (unsigned)workgroup);
   const unsigned end = sk_first_unit(sp, (unsigned)workgroup + 1);
+  unsigned whole = (unsigned)workgroup;
   int n = 0;
-  while (unit < end) {
-    const sk_segment seg = sk_segment_at(sp, unit, end);
-    unit += seg.ke - seg.kb;
+  while (unit < end || whole < sp.dp_tiles) {
+    sk_segment seg;
+    if (unit < end) {
+      seg = sk_segment_at(sp, unit, end);
+      unit += seg.ke - seg.kb;
+    } else {
+      seg = sk_whole_tile(sp, whole);
+      whole += sp.grid;
+    }
     if (n < capacity) {
       rl_streamk_segment& o = out[n];
       o.tile = (int)seg.tile; o.tile_m = (int)seg.tile_m; o.tile_n = (int)seg.tile_n;
       o.k_begin = (int)seg.kb; o.k_end = (int)seg.ke;
       o.pieces = 1; o.first_workgroup = workgroup; o.slot = -1;
       if (seg.kb != 0 || seg.ke != sp.kt) {
-        const unsigned first_wg = sk_owner(sp, seg.tile * sp.kt);
+        const unsigned first_wg = sk_owner(sp, sk_tile_unit(sp, seg.tile));
         o.first_workgroup = (int)first_wg;
-        o.pieces = (int)(sk_owner(sp, seg.tile * sp.kt + sp.kt - 1) - first_wg + 1);
+        o.pieces = (int)(sk_owner(sp, sk_tile_unit(sp, seg.tile) + sp.kt - 1) - first_wg + 1);
         o.slot = 2 * workgroup + (seg.kb == 0 ? 1 : 0);
       }
     }

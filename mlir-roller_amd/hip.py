@@ -68,7 +68,7 @@ class _GemmConfigC(C.Structure):
 class StreamKSchedule(C.Structure):
     """``rl_streamk_schedule``: how a stream-K configuration splits one problem."""
     _fields_ = [("grid", C.c_int), ("k_steps", C.c_int), ("tiles", C.c_int), ("tile_rows", C.c_int), ("tile_cols", C.c_int),
-                ("units", C.c_long), ("workspace_bytes", C.c_size_t), ("counter_bytes", C.c_size_t)]
+                ("units", C.c_long), ("workspace_bytes", C.c_size_t), ("counter_bytes", C.c_size_t), ("whole_tiles", C.c_int)]
 
 
 class StreamKSegment(C.Structure):

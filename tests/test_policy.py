@@ -372,7 +372,7 @@ def test_mi355x_top_hints_compile_without_spills_or_scratch():
         # segments of a workgroup; their K loop itself carries no such traffic, which a GPU timing shows)
         # -- and the kernels for dword-aligned rows (the step that K ends in works its offsets out again)
         assert res["sgpr_spills"] == 0 or (res["sgpr_spills"] <= 64 and (g.threads == 64 or g.streamk)) \
-            or (res["sgpr_spills"] <= 128 and g.vec == 1), (shape, g.tag(), res)
+            or (res["sgpr_spills"] <= 160 and g.vec == 1), (shape, g.tag(), res)
         assert 0 < res["vgprs"] <= 512 // max(1, g.threads // 256), (g.tag(), res)
         # a stream-K grid is sized for that many workgroups per CU: they have to fit the register file together
         if g.streamk and g.threads >= 256:

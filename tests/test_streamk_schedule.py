@@ -2,9 +2,10 @@
 
 ``rl_gemm_streamk_segments`` runs, for one workgroup index, the very code the kernel's workgroups run
 (csrc/gemm_sk_decode.inc is compiled into the library and into every stream-K kernel).  Walking all
-workgroups of a launch must hand out every K step of every tile exactly once, in pieces that belong
-to consecutive workgroups in K order, each in a workspace slot of its own -- which is what makes the
-sum of a split tile independent of which workgroup finishes last."""
+workgroups of a launch must hand out every K step of every tile exactly once: the first rounds of
+tiles whole, one tile per workgroup and round (neighbouring tiles at the same time), the rest in pieces
+that belong to consecutive workgroups in K order, each in a workspace slot of its own -- which is what
+makes the sum of a split tile independent of which workgroup finishes last."""
 
 import random
 
@@ -40,6 +41,9 @@ CASES = [
     (sk_config(128, 64, 32, 64, 32, 16, 2, group=3), (1100, 900, 512), 7),   # odd CU count, short last panel
     (sk_config(128, 64, 32, 64, 32, 16, 2, swz=1), (1100, 900, 512), 304),
     (sk_config(96, 96, 32, 48, 48, 16, 2), (96 * 5 + 1, 96 * 7 + 95, 32 * 9), 16),
+    (sk_config(128, 96, 32, 64, 48, 16, 1), (4095, 4097, 4093), 256),        # 1376 tiles on 512 workgroups: one round whole, 864 tiles shared
+    (sk_config(64, 160, 32, 32, 80, 16, 0), (8192, 8192, 8192), 256),        # 6656 tiles = 13 rounds, nothing shared
+    (sk_config(64, 64, 32, 32, 32, 16, 1, streamk=1), (1000, 1000, 1000), 60),   # 256 tiles on 60: three rounds whole, 76 tiles shared
 ]
 
 
@@ -55,16 +59,25 @@ def test_every_k_step_of_every_tile_is_handed_out_once(lib, cfg, shape, cus):
     nbm, nbn, kt = -(-M // cfg.bm), -(-N // cfg.bn), -(-K // cfg.bk)
     assert (sched.tile_rows, sched.tile_cols, sched.k_steps, sched.tiles, sched.units) == (nbm, nbn, kt, nbm * nbn, nbm * nbn * kt)
     assert sched.grid == min(cus * cfg.streamk, sched.units)
+    # all rounds of whole tiles but the last are worked whole (every round, if the last is a full one too)
+    rounds = sched.tiles // sched.grid
+    assert sched.whole_tiles == sched.grid * (rounds if rounds and sched.tiles % sched.grid == 0 else max(rounds - 1, 0))
     covered, tile_number, pieces_of = {}, {}, {}
     for wg, segs in enumerate(per_wg):
         assert segs, f"workgroup {wg} has no work"            # the decoding of pieces relies on it
+        # its share of the tiles that are shared out comes first, then its whole tiles: tile round * grid + wg
+        shared = [s for s in segs if s.tile >= sched.whole_tiles]
+        assert [s.tile for s in segs[:len(shared)]] == [s.tile for s in shared]
+        assert [(s.tile, s.k_begin, s.k_end, s.pieces) for s in segs[len(shared):]] == \
+            [(t, 0, kt, 1) for t in range(wg, sched.whole_tiles, sched.grid)]
+        assert bool(shared) == (sched.whole_tiles < sched.tiles)
         for i, s in enumerate(segs):
             assert 0 <= s.tile_m < nbm and 0 <= s.tile_n < nbn and 0 <= s.k_begin < s.k_end <= kt
             assert tile_number.setdefault((s.tile_m, s.tile_n), s.tile) == s.tile and 0 <= s.tile < sched.tiles
             for k in range(s.k_begin, s.k_end):
                 assert (s.tile_m, s.tile_n, k) not in covered
                 covered[(s.tile_m, s.tile_n, k)] = wg
-            pieces_of.setdefault((s.tile_m, s.tile_n), []).append((wg, i, len(segs), s))
+            pieces_of.setdefault((s.tile_m, s.tile_n), []).append((wg, i, len(shared), s))
     assert len(covered) == nbm * nbn * kt                       # nothing left out ...
     assert sum(s.k_end - s.k_begin for segs in per_wg for s in segs) == nbm * nbn * kt   # ... and nothing twice
     assert len(set(tile_number.values())) == nbm * nbn          # one arrival counter per tile
@@ -86,7 +99,7 @@ def test_every_k_step_of_every_tile_is_handed_out_once(lib, cfg, shape, cus):
                 assert s.slot not in used_slots and 0 <= s.slot < 2 * sched.grid
                 used_slots.add(s.slot)
                 # a piece that starts inside a tile is its workgroup's first segment; one that starts a
-                # tile and does not finish it is its last
+                # tile and does not finish it is the last of its share
                 assert (i == 0) if s.k_begin else (i == n - 1)
     assert sched.workspace_bytes == sched.counter_bytes + 2 * sched.grid * cfg.bm * cfg.bn * 4
     assert sched.counter_bytes >= 4 * sched.tiles and sched.counter_bytes % 256 == 0
@@ -102,12 +115,11 @@ def test_shares_are_equal_to_within_one_k_step(lib, cfg, shape, cus):
 def test_tiles_are_walked_in_panels(lib):
     # panel of 3 tile rows over a 9 x 15 tile grid: consecutive tiles go down a panel's column first
     cfg = sk_config(128, 64, 32, 64, 32, 16, 2, group=3)
-    order = []
+    where = {}
     for wg in range(hip.streamk_schedule(cfg, 1100, 900, 512, 7).grid):
         for s in hip.streamk_segments(cfg, 1100, 900, 512, wg, 7):
-            if (s.tile_m, s.tile_n) not in order:
-                order.append((s.tile_m, s.tile_n))
-                assert s.tile == len(order) - 1
+            assert where.setdefault(s.tile, (s.tile_m, s.tile_n)) == (s.tile_m, s.tile_n)
+    order = [where[t] for t in range(len(where))]
     assert order[:7] == [(0, 0), (1, 0), (2, 0), (0, 1), (1, 1), (2, 1), (0, 2)] and order[45] == (3, 0) and len(order) == 9 * 15
 
 
