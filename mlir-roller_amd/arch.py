@@ -153,11 +153,11 @@ class MI355X(TileDevice):
     peak_matrix_tflops: float = 157.3
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
-    # (a test refits them): 0.979 for 256x256 tiles, 0.974 + 0.006 for 128x128 with two on a CU,
-    # 0.969 + 0.006 for 64x128; below that knee the efficiency falls 2.4 per unit of (1/m + 1/n)
-    # faster (0.945 for 64x64, 0.90 for 32x64)
-    mfma_efficiency: Tuple[float, float] = (0.984, 0.66)
-    co_resident_gain: float = 0.006
+    # (a test refits them): 0.981 for 256x256 tiles, 0.976 + 0.007 for 128x128 with two on a CU,
+    # 0.971 + 0.007 for 64x128; below that knee the efficiency falls 2.4 per unit of (1/m + 1/n)
+    # faster (0.95 for 64x64, 0.90 for 32x64)
+    mfma_efficiency: Tuple[float, float] = (0.986, 0.62)
+    co_resident_gain: float = 0.007
     small_tile_slope: float = 2.4
     tile_fixed_seconds: float = 1.0e-6
     # chosen on the committed sweep, not fitted in closed form: 0.2-0.4 us and ratios of 2.5-4 rank
@@ -173,12 +173,12 @@ class MI355X(TileDevice):
     # tiles at K steps of 32 against 64, 64x64 at 32 / 64 / 128: the shortest wins or ties)
     grow_reduce_step: bool = False
     # fitted like the constants above: stream-K against plain kernels of the same tile on problems that
-    # fill whole rounds (0.6 % slower), and the rate at which the last workgroup of a tile that is split
-    # many ways reads the pieces back (35 GB/s: a round trip past the L2 each); about 5 us per launch besides
+    # fill whole rounds (0.5 % slower), and the rate at which the last workgroup of a tile that is split
+    # many ways reads the pieces back (32 GB/s: a round trip past the L2 each); about 5 us per launch besides
     stream_k_workgroups: int = 2
-    stream_k_loss: float = 0.006
+    stream_k_loss: float = 0.005
     stream_k_fixed_seconds: float = 5.0e-6
-    stream_k_piece_bandwidth: float = 35.0
+    stream_k_piece_bandwidth: float = 32.0
     stream_k_margin: float = 0.02
     smem_cap: int = field(init=False)
     max_smem_usage: int = field(init=False)

@@ -92,6 +92,40 @@ def test_streamk_matches_oracle_within_tolerance_and_exactly_on_integers(device,
         assert np.array_equal(first.view(np.uint32), run(cfg, A, B).view(np.uint32))   # same bits whoever arrives last
 
 
+# (config, shape, rounds of whole tiles, tiles shared out) on 256 CUs
+ROUNDS = [
+    (GemmConfig(32, 32, 32, 16, 16, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1, 0, 2), (1500, 1300, 200), 2, 903),    # 1927 tiles on 512 workgroups
+    (GemmConfig(32, 32, 32, 16, 16, 16, 3, 0, 0, 4, 0, 3, 8, 0, 1, 0, 2), (1024, 1024, 96), 2, 0),       # two full rounds, nothing split
+    (GemmConfig(32, 32, 32, 16, 16, 16, 3, 0, 0, 4, 1, 3, 8, 0, 1, 0, 2), (1600, 1632, 72), 3, 1014),
+    (GemmConfig(64, 64, 32, 32, 32, 16, 3, 0, 0, 1, 1, 3, 8, 0, 1, 0, 2), (2049, 2047, 131), 1, 544),    # dword-aligned rows
+    (GemmConfig(64, 32, 32, 16, 32, 16, 3, 0, 0, 4, 2, 0, 8, 0, 1, 1, 1), (1000, 1100, 160), 1, 304),    # no remap, Bt, 560 tiles on 256
+    (GemmConfig(32, 64, 32, 16, 32, 16, 3, 0, 0, 4, 2, 2, 5, 1, 1, 0, 4), (3100, 2100, 64), 2, 1153),    # panels of 5, accumulate, 3201 tiles on 1024
+]
+
+
+@pytest.mark.parametrize("cfg,shape,rounds,shared", ROUNDS, ids=[f"{c.tag()}-{s[0]}x{s[1]}x{s[2]}" for c, s, _, _ in ROUNDS])
+def test_rounds_of_whole_tiles_and_a_shared_remainder(device, cfg, shape, rounds, shared):
+    """From two tiles per workgroup on, a stream-K launch works all rounds of its grid but the last as
+    whole tiles and shares out the K steps of the rest: exact on integers and the same bits every run."""
+    M, N, K = shape
+    sched = hip.streamk_schedule(cfg, M, N, K, device.compute_units)
+    say("case", cfg.tag(), shape, "grid", sched.grid, "tiles", sched.tiles, "whole", sched.whole_tiles)
+    if device.compute_units == 256:
+        assert (sched.whole_tiles, sched.tiles - sched.whole_tiles) == (rounds * sched.grid, shared)
+    A, B = go.make_inputs(M, N, K, seed=5, distribution="integer")
+    want = host_gemm(A, B)
+    if cfg.accum:
+        C0 = np.random.default_rng(3).integers(-9, 9, (M, N)).astype(np.float32)
+        assert np.array_equal(run(cfg, A, B, c_init=C0), want + C0)
+    else:
+        assert np.array_equal(run(cfg, A, B), want)
+        assert np.array_equal(run(cfg, A, B), want)
+        A, B = go.make_inputs(M, N, K, seed=6)
+        first = run(cfg, A, B)
+        assert go.error_report(first, A, B)["ok"]
+        assert np.array_equal(first.view(np.uint32), run(cfg, A, B).view(np.uint32))
+
+
 def test_seeded_points_of_the_template_parameter_space_are_exact_as_stream_k(device):
     """Forty-eight seeded (configuration, shape) pairs from everything the configuration check accepts with
     ``streamk`` set -- both instructions, 1 to 8 waves, 1 to 7 column blocks per wave, both operand layouts,
