@@ -661,11 +661,27 @@ class Policy:
         the kernel, whole tiles or stream-K, where the estimate cannot tell the two apart."""
         rstep = self._assign_reduce_step()
         hints: List[TileDict] = []
+        late: List[Tuple[float, TileDict]] = []
         mfma = self.arch.has_matrix_cores
         for td in self.get_block_tiles_candidates([1, 1], rstep):
             self._expand_reduce_axis(td)
+            # hints that lost their place when their wave tile was assigned (below) come back in
+            # where their estimate puts them
+            ranked = self._priority(td) if mfma else 0.0
+            while late and late[0][0] <= ranked and len(hints) < topk:
+                hints.append(late.pop(0)[1])
+            if len(hints) >= topk:
+                return hints[:topk]
             for hint in self.assign_thread_tile(td, 1 if mfma else 2):
                 hint.stream_k = self._stream_k_fit(hint, hint.stream_k)
+                if mfma and (hint.block_per_SM != td.block_per_SM or hint.stream_k != td.stream_k):
+                    # the tile was ranked as if more of its workgroups shared a core than the registers
+                    # of this wave tile allow: rank it again by what it is now expected to take
+                    now = self.estimate_seconds(hint)
+                    if now > ranked:
+                        late.append((now, hint))
+                        late.sort(key=lambda e: e[0])
+                        continue
                 hints.append(hint)
                 if mfma and self.arch.stream_k_workgroups and 2 <= self.pipeline_depth <= 3:
                     other = self._stream_k_fit(hint, max(1, min(self.arch.stream_k_workgroups, hint.block_per_SM))) if not hint.stream_k else 0
@@ -676,7 +692,7 @@ class Policy:
                         hints.append(twin)
                 if len(hints) >= topk:
                     return hints[:topk]
-        return hints
+        return (hints + [hint for _, hint in late])[:topk]
 
 
 def get_roller_hints(matmul_config: MatmulConfig, arch: TileDevice, topk: int = 10,
