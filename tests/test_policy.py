@@ -442,6 +442,31 @@ def test_committed_ranking_constants_equal_a_refit_of_the_committed_sweep():
         assert rows[shape]["top1_over_fastest"] <= 1.02, rows[shape]
 
 
+def test_first_four_hints_on_dword_aligned_shapes_hold_a_kernel_within_a_percent_and_a_half_of_the_fastest():
+    """Shapes whose K or N is not a multiple of 4 (rows that are only dword-aligned) have a data set of
+    their own, measured like the sweep (``calibrate measure --shapes ... --out``): seven shapes from
+    1001 x 999 x 1003 to 8191 x 8193 x 8189, 96 kernels each in both forms.  No constant is fitted to it;
+    it checks that the model that was fitted to aligned shapes still orders these: whole tiles of 64 x 96,
+    four to a CU, are the fastest kernel on five of them (the loads of misaligned rows touch two cache
+    lines where aligned ones touch one, and more resident workgroups hide that), stream-K kernels on big
+    tiles come next, and a workgroup of more than 256 registers (128 x 160 with the 60 registers that
+    dword-aligned rows cost) is known to run alone."""
+    from mlir_roller_amd import calibrate
+    data = calibrate.load(calibrate.DATA_DIR / "mi355x_f32_dword_rows.json")
+    records = data["records"]
+    shapes = {tuple(r["shape"]) for r in records}
+    assert len(shapes) == 7 and all(s[1] % 4 or s[2] % 4 for s in shapes) and len(records) >= 600
+    rows = {tuple(r["shape"]): r for r in calibrate.check(records, topk=4)}
+    for shape, row in rows.items():
+        assert row["unmeasured_in_topk"] == 0 and row["topk_over_fastest"] <= 1.015, row
+        assert row["top1_over_fastest"] <= 1.07, row
+    fastest = {s: min((r for r in records if tuple(r["shape"]) == s), key=lambda r: r["ms"]) for s in shapes}
+    assert sum(1 for r in fastest.values() if sorted(r["block_tile"]) == [64, 96] and not r["stream_k"]) >= 4
+    # 4095 x 4097 x 4093 runs at 0.92 of the matrix peak, its aligned neighbour 4096^3 at 0.97
+    best = fastest[(4095, 4097, 4093)]["ms"]
+    assert 2.0 * 4095 * 4097 * 4093 / best / 1e9 > 0.9 * MI355X().peak_matrix_tflops
+
+
 def test_the_latency_and_cache_terms_of_the_estimate_matter_where_k_is_long_and_tiles_are_few():
     """``step_latency_seconds`` and ``cache_bandwidth_ratio`` are not fitted in closed form but chosen on
     the committed sweep; this pins what they are for.  With both switched off the first four hints of
