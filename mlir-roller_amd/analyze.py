@@ -435,20 +435,20 @@ class Policy:
         return tiles_per_cu * max(t_mfma, t_mem) + (-(-tiles_per_cu // resident)) * t_fixed
 
     def stream_k_pieces(self, td: TileDict, stream_k: int) -> float:
-        """How many workgroups meet in one split tile of a stream-K launch.  From two tiles per workgroup
-        on, all rounds of the grid but the last are worked as whole tiles (all of them, if the tile count
-        is a multiple of the grid: nothing is split then) and the reduce steps of the remaining tiles are
-        shared out: a share is at least a tile long and ends inside at most one tile, two pieces.  With
-        fewer tiles everything is shared out, and with fewer reduce steps in a share than in a tile a
-        tile has its steps / a share's steps pieces, plus one for the share that straddles its start.
+        """How many workgroups meet in one split tile of a stream-K launch.  The full rounds of the grid
+        are worked as whole tiles (all but one of them, if fewer tiles than a quarter of the grid are
+        left over) and the reduce steps of the remaining tiles are shared out: a share that is at least
+        a tile long ends inside at most one tile, two pieces; with fewer reduce steps in a share than in
+        a tile a tile has its steps / a share's steps pieces, plus one for the share that straddles its
+        start; nothing is split if the grid divides the tile count.
         The workgroup that arrives last reads that many pieces of the tile back, one after the other,
         which is what a split costs."""
         k_steps = -(-self.matmul_config.K // td.rstep)
         tiles = td.grid_size
         grid = min(stream_k * self.arch.compute_max_core, tiles * k_steps)
-        rounds = tiles // grid - 1 if tiles >= 2 * grid else 0
-        if tiles >= grid and tiles % grid == 0:
-            rounds = tiles // grid
+        rounds = tiles // grid
+        if rounds and tiles % grid and ((tiles % grid) * 4 < grid or (tiles % grid) * k_steps < grid):
+            rounds -= 1
         units = (tiles - rounds * grid) * k_steps
         if not units:
             return 0.0

@@ -421,9 +421,8 @@ sk_div make_div(unsigned d) {
 
 // Fills *p for cfg on an M x N x K problem with `compute_units` CUs.  The grid is cfg.streamk
 // workgroups per CU, cut down to one K step per workgroup where the problem is smaller than that
-// (the decoding relies on no share being empty, unless all are).  From two tiles per workgroup on,
-// all rounds of whole tiles but the last are worked as whole tiles (all of them if the tile count is
-// a multiple of the grid) and only the units of the remaining tiles are shared out.
+// (the decoding relies on no share being empty, unless all are).  Full rounds of the grid are worked
+// as whole tiles and only the units of the remaining tiles are shared out.
 int sk_make_params(const rl_gemm_config& c, int M, int N, int K, int compute_units, sk_params* p, unsigned* tiles) {
   if (!c.streamk) return fail(RL_ERR_INVALID_ARG, "not a stream-K configuration");
   if (M <= 0 || N <= 0 || K <= 0) return fail(RL_ERR_INVALID_ARG, "stream-K needs M, N, K > 0 (M=%d N=%d K=%d)", M, N, K);
@@ -436,8 +435,11 @@ int sk_make_params(const rl_gemm_config& c, int M, int N, int K, int compute_uni
   unsigned long grid = (unsigned long)compute_units * c.streamk;
   if (grid > units) grid = units;
   const unsigned long n_tiles = nbm * nbn;
-  unsigned long rounds = n_tiles >= 2 * grid ? n_tiles / grid - 1 : 0;
-  if (n_tiles >= grid && n_tiles % grid == 0) rounds = n_tiles / grid;
+  // rounds of whole tiles: all full rounds if the tiles left over are at least a quarter of a round (a
+  // tile of theirs is then split four or five ways at most) and no share is empty; else all but one
+  // (shares of more than a tile)
+  unsigned long rounds = n_tiles / grid;
+  if (rounds && (n_tiles % grid) && ((n_tiles % grid) * 4 < grid || (n_tiles % grid) * kt < grid)) --rounds;
   const unsigned long shared = (n_tiles - rounds * grid) * kt;   // units that are shared out
   memset(p, 0, sizeof *p);
   p->grid = (unsigned)grid; p->dp_tiles = (unsigned)(rounds * grid);

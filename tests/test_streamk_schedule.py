@@ -2,7 +2,7 @@
 
 ``rl_gemm_streamk_segments`` runs, for one workgroup index, the very code the kernel's workgroups run
 (csrc/gemm_sk_decode.inc is compiled into the library and into every stream-K kernel).  Walking all
-workgroups of a launch must hand out every K step of every tile exactly once: the first rounds of
+workgroups of a launch must hand out every K step of every tile exactly once: the full rounds of
 tiles whole, one tile per workgroup and round (neighbouring tiles at the same time), the rest in pieces
 that belong to consecutive workgroups in K order, each in a workspace slot of its own -- which is what
 makes the sum of a split tile independent of which workgroup finishes last."""
@@ -41,9 +41,9 @@ CASES = [
     (sk_config(128, 64, 32, 64, 32, 16, 2, group=3), (1100, 900, 512), 7),   # odd CU count, short last panel
     (sk_config(128, 64, 32, 64, 32, 16, 2, swz=1), (1100, 900, 512), 304),
     (sk_config(96, 96, 32, 48, 48, 16, 2), (96 * 5 + 1, 96 * 7 + 95, 32 * 9), 16),
-    (sk_config(128, 96, 32, 64, 48, 16, 1), (4095, 4097, 4093), 256),        # 1376 tiles on 512 workgroups: one round whole, 864 tiles shared
+    (sk_config(128, 96, 32, 64, 48, 16, 1), (4095, 4097, 4093), 256),        # 1376 tiles on 512 workgroups: two rounds whole, 352 tiles shared
     (sk_config(64, 160, 32, 32, 80, 16, 0), (8192, 8192, 8192), 256),        # 6656 tiles = 13 rounds, nothing shared
-    (sk_config(64, 64, 32, 32, 32, 16, 1, streamk=1), (1000, 1000, 1000), 60),   # 256 tiles on 60: three rounds whole, 76 tiles shared
+    (sk_config(64, 64, 32, 32, 32, 16, 1, streamk=1), (1000, 1000, 1000), 60),   # 256 tiles on 60: four rounds whole, 16 tiles shared
 ]
 
 
@@ -59,9 +59,10 @@ def test_every_k_step_of_every_tile_is_handed_out_once(lib, cfg, shape, cus):
     nbm, nbn, kt = -(-M // cfg.bm), -(-N // cfg.bn), -(-K // cfg.bk)
     assert (sched.tile_rows, sched.tile_cols, sched.k_steps, sched.tiles, sched.units) == (nbm, nbn, kt, nbm * nbn, nbm * nbn * kt)
     assert sched.grid == min(cus * cfg.streamk, sched.units)
-    # all rounds of whole tiles but the last are worked whole (every round, if the last is a full one too)
-    rounds = sched.tiles // sched.grid
-    assert sched.whole_tiles == sched.grid * (rounds if rounds and sched.tiles % sched.grid == 0 else max(rounds - 1, 0))
+    # the full rounds of the grid are worked whole -- all but one if the tiles left over are fewer than a
+    # quarter of the grid (or have fewer K steps than there are workgroups)
+    rounds, left = divmod(sched.tiles, sched.grid)
+    assert sched.whole_tiles == sched.grid * (rounds - 1 if rounds and left and (4 * left < sched.grid or left * kt < sched.grid) else rounds)
     covered, tile_number, pieces_of = {}, {}, {}
     for wg, segs in enumerate(per_wg):
         assert segs, f"workgroup {wg} has no work"            # the decoding of pieces relies on it
