@@ -651,7 +651,7 @@ class Policy:
     # ---- top level ------------------------------------------------------------------------------
 
     # a block tile whose plain and stream-K estimates are this close is emitted in both forms
-    STREAM_K_TOSS_UP = 0.005
+    STREAM_K_TOSS_UP = 0.002
 
     def emit_config(self, topk: int = 10) -> List[TileDict]:
         """The first ``topk`` hints.  The reference completes every block tile with its first two

@@ -153,12 +153,12 @@ class MI355X(TileDevice):
     peak_matrix_tflops: float = 157.3
     clock_mhz: int = 2400
     # fitted to the committed sweep under calibration/ by ``python -m mlir_roller_amd.calibrate fit``
-    # (a test refits them): 0.981 for 256x256 tiles, 0.976 + 0.007 for 128x128 with two on a CU,
-    # 0.971 + 0.007 for 64x128; below that knee the efficiency falls 2.4 per unit of (1/m + 1/n)
-    # faster (0.95 for 64x64, 0.90 for 32x64)
-    mfma_efficiency: Tuple[float, float] = (0.986, 0.62)
+    # (a test refits them): 0.980 for 256x256 tiles, 0.974 + 0.007 for 128x128 with two on a CU,
+    # 0.968 + 0.007 for 64x128; below that knee the efficiency falls 2.7 per unit of (1/m + 1/n)
+    # faster (0.94 for 64x64, 0.89 for 32x64)
+    mfma_efficiency: Tuple[float, float] = (0.986, 0.75)
     co_resident_gain: float = 0.007
-    small_tile_slope: float = 2.4
+    small_tile_slope: float = 2.7
     tile_fixed_seconds: float = 1.0e-6
     # chosen on the committed sweep, not fitted in closed form: 0.2-0.4 us and ratios of 2.5-4 rank
     # its kernels identically (a test holds both ends); without the two, whole tiles of 32 x 32 lead on
@@ -173,12 +173,12 @@ class MI355X(TileDevice):
     # tiles at K steps of 32 against 64, 64x64 at 32 / 64 / 128: the shortest wins or ties)
     grow_reduce_step: bool = False
     # fitted like the constants above: stream-K against plain kernels of the same tile on problems that
-    # fill whole rounds (0.5 % slower), and the rate at which the last workgroup of a tile that is split
-    # many ways reads the pieces back (32 GB/s: a round trip past the L2 each); about 5 us per launch besides
+    # fill whole rounds (0.3 % slower), and the rate at which the last workgroup of a tile that is split
+    # many ways reads the pieces back (33 GB/s: a round trip past the L2 each); about 5 us per launch besides
     stream_k_workgroups: int = 2
-    stream_k_loss: float = 0.005
+    stream_k_loss: float = 0.003
     stream_k_fixed_seconds: float = 5.0e-6
-    stream_k_piece_bandwidth: float = 32.0
+    stream_k_piece_bandwidth: float = 33.0
     stream_k_margin: float = 0.02
     smem_cap: int = field(init=False)
     max_smem_usage: int = field(init=False)

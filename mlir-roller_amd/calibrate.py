@@ -501,10 +501,11 @@ def main(argv=None) -> int:
         print(f"{len(set(todo))} kernels, {len(failed)} failed to compile")
         return 1 if failed else 0
     if args.cmd == "measure":
+        earlier_sets = [load(Path(earlier)) for earlier in args.merge]   # (read first: a missing file should not cost a session)
         data = measure(args.shapes, args.topk)
         data["sessions"] = 1
-        for earlier in args.merge:
-            data = merge(data, load(Path(earlier)))
+        for earlier in earlier_sets:
+            data = merge(data, earlier)
         out = Path(args.out)
         out.parent.mkdir(parents=True, exist_ok=True)
         out.write_text(json.dumps(data, separators=(",", ":")).replace('},{"shape"', '},\n{"shape"'))
