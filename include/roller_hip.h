@@ -81,9 +81,9 @@ typedef struct rl_gemm_config {
                       layout of MatmulConfig.get_input_shapes, src/analyze.py:33-41); pad_b then
                       pads the K-contiguous rows of its LDS tile like pad_a                   */
   int streamk;     /* 0: one workgroup per tile of C, grid (ceil(N/bn), ceil(M/bm)) as at src/roller.py:536.
-                      1..8: a fixed grid of that many workgroups per CU; each works an equal share of all
-                      (tile, K step) units, and tiles whose K range is split are summed in K order through
-                      a workspace.  Stands in for what the reference gets from ranking tilings by rounds of
+                      1..8: a fixed grid of that many workgroups per CU; each works one tile of every full
+                      round of the grid and an equal share of the (tile, K step) units of the tiles left
+                      over, and tiles whose K range is split are summed in K order through a workspace.  Stands in for what the reference gets from ranking tilings by rounds of
                       blocks (num_wave, src/analyze.py:164-166).  Needs stages=3                     */
 } rl_gemm_config;
 

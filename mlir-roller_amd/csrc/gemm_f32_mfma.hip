@@ -561,10 +561,9 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
 
 #if DIRECT
   // Issues the loads of K step kt straight into LDS buffer `stage`.  Instruction i of a wave
-  // fills the 64 consecutive 16-byte units (floats, with dword-aligned rows) that start at unit
-  // i*NT + wave*64 of the operand tile.
+  // fills the 64 consecutive 16-byte units that start at unit i*NT + wave*64 of the operand tile.
   // KTAIL (a compile-time 0/1) says whether tile kt may be the one that K ends in: only then are
-  // the units tested against K.
+  // the units tested against K (with dword-aligned rows: is the tile loaded float by float).
   auto fetch_direct = [&](auto ktail, int kt, int stage) __attribute__((always_inline)) {
     constexpr bool KTEST = EDGE_K && decltype(ktail)::value;
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -811,12 +810,11 @@ extern "C" __global__ __launch_bounds__(NT) void gemm_kernel(
     // P = which of the two fragment sets holds round 0 of this step (compile-time, so that the
     // sets stay in fixed registers); the set alternates every round.
     // MFMAs and fragment reads per round; LDS writes and global loads per K step
-    constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NSEG), W = A_PER_T + B_PER_T, L0 = DIRECT ? LOADS_PER_TILE : W * (VEC == 4 ? 1 : 4);
+    constexpr int G = 4 * TM * TN, R = TM + (TRANS_B ? TN : 4 * NSEG), W = A_PER_T + B_PER_T, L = DIRECT ? LOADS_PER_TILE : W * (VEC == 4 ? 1 : 4);
 
     // `buffer`: the LDS buffer of this step's tile when there are two (with more, kt % LDS_BUFS).
     auto step = [&](auto parity, auto ktail, auto buffer, int kt) __attribute__((always_inline)) {
       constexpr int P = decltype(parity)::value;
-      constexpr int L = L0;
       const int cur = LDS_BUFS == 2 ? decltype(buffer)::value : (unsigned)kt % LDS_BUFS;
       const int nxt = LDS_BUFS == 2 ? 1 - decltype(buffer)::value : (unsigned)(kt + 1) % LDS_BUFS;
 #pragma unroll
