@@ -341,6 +341,35 @@ def test_leading_dimensions_wider_than_the_matrix(device):
     assert np.all(out[:, N:] == -7.0)                               # padding columns untouched
 
 
+def test_dword_aligned_views_with_odd_offsets_and_leading_dimensions(device):
+    """Sub-matrices that start at odd float offsets inside larger buffers, with odd leading dimensions:
+    every row of A, B and C is only dword-aligned, and differently so from row to row.  Through the
+    direct-to-LDS kernels for dword-aligned rows -- whole tiles, stream-K, and the Bt layout -- the
+    result is exact and nothing outside the C view is touched."""
+    M, N, K, lda, ldb, ldc = 203, 299, 1037, 1051, 307, 311
+    rng = np.random.default_rng(22)
+    A, B = go.make_inputs(M, N, K, seed=23, distribution="integer")
+    want = go.gemm_f32(A, B)
+    for cfg in (GemmConfig(128, 128, 32, 64, 64, 16, 3, 0, 0, 1, 1, 3, 8, 0, 1, 0, 0),
+                GemmConfig(64, 96, 32, 32, 48, 16, 3, 0, 0, 1, 1, 3, 8, 0, 1, 0, 2),
+                GemmConfig(64, 64, 32, 32, 32, 32, 3, 0, 0, 1, 1, 3, 8, 0, 1, 1, 0)):
+        say("views", cfg.tag())
+        second = np.ascontiguousarray(B.T) if cfg.trans_b else B            # Bt[N][ldb >= K] or B[K][ldb >= N]
+        rows_b, width_b = second.shape
+        ld_b = 1049 if cfg.trans_b else ldb
+        hA = rng.integers(0, 10, (M * lda + 3,)).astype(np.float32)        # the views start 3, 1 and 5 floats in
+        hB = rng.integers(0, 10, (rows_b * ld_b + 1,)).astype(np.float32)
+        hC = np.full((M * ldc + 5,), -7.0, np.float32)
+        hA[3:].reshape(M, lda)[:, :K] = A
+        hB[1:].reshape(rows_b, ld_b)[:, :width_b] = second
+        dA, dB, dC = DeviceArray.from_host(hA), DeviceArray.from_host(hB), DeviceArray.from_host(hC)
+        GemmPlan(cfg).launch(hip.Ptr(dA.ptr + 12), hip.Ptr(dB.ptr + 4), hip.Ptr(dC.ptr + 20), M, N, K, lda, ld_b, ldc)
+        hip.synchronize()
+        out = dC.get()
+        assert np.array_equal(out[5:].reshape(M, ldc)[:, :N], want), cfg.tag()
+        assert np.all(out[:5] == -7.0) and np.all(out[5:].reshape(M, ldc)[:, N:] == -7.0), cfg.tag()   # nothing beside the view
+
+
 def test_empty_and_zero_k(device):
     plan = GemmPlan(GemmConfig(128, 128, 16, 64, 64, 32, 2, 4, 0, 4, 1))
     dC = DeviceArray.from_host(np.full((8, 12), 3.0, np.float32))
