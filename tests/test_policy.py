@@ -472,6 +472,30 @@ def test_first_four_hints_on_dword_aligned_shapes_hold_a_kernel_close_to_the_fas
     assert 2.0 * 4095 * 4097 * 4093 / best / 1e9 > 0.9 * MI355X().peak_matrix_tflops
 
 
+def test_a_hint_that_loses_its_residency_is_ranked_again():
+    """Block tiles are ranked before their wave tile is known.  On 8191 x 8193 x 8189 (dword-aligned rows: 60
+    more registers) the 128 x 160 tile is ranked as two workgroups per CU, and its wave tile of 64 x 80 then
+    turns out to need more than half of the register file: the hint is emitted where its new estimate puts
+    it, not where the tile stood, and a stream-K form never asks for more workgroups than fit."""
+    arch = MI355X()
+    cfg = MatmulConfig(8191, 8193, 8189, 32)
+    policy = Policy(cfg, arch)
+    hints = get_roller_hints(cfg, arch, topk=12)
+    alone = [h for h in hints if h.block_tile == [128, 160]]
+    assert alone and all(h.block_per_SM == 1 and h.stream_k <= 1 for h in alone)
+    assert TileDict.from_block_tile([128, 160], 32, cfg, arch).block_per_SM == 2           # as the tile was ranked
+    first = [policy.estimate_seconds(h) for h in hints[:4]]
+    assert max(first) <= min(policy.estimate_seconds(h) for h in hints) * 1.005            # nothing cheaper was pushed out of the first four
+    assert not any(h.block_tile == [128, 160] for h in hints[:4])
+    for h in hints:
+        if h.stream_k and h.threads >= 256:
+            regs = int(h.wave_tile[0] * h.wave_tile[1] // 64) + policy._reg_overhead(h, h.wave_tile, h.mfma, h.threads)
+            assert h.stream_k * (h.threads // 256) * regs <= arch.regs_per_lane, (h.block_tile, h.stream_k, regs)
+    # an aligned neighbour keeps the tile at two per CU
+    aligned = get_roller_hints(MatmulConfig(8192, 8192, 8192, 32), arch, topk=12)
+    assert all(h.block_per_SM == 2 for h in aligned if h.block_tile == [128, 160])
+
+
 def test_the_latency_and_cache_terms_of_the_estimate_matter_where_k_is_long_and_tiles_are_few():
     """``step_latency_seconds`` and ``cache_bandwidth_ratio`` are not fitted in closed form but chosen on
     the committed sweep; this pins what they are for.  With both switched off the first four hints of
